@@ -13,8 +13,11 @@ import math
 import torch
 
 
-def embed(token_ids, table):
-    return table[token_ids.long()].to(torch.float32)
+def embed(token_ids, table, positions=None, position_table=None):
+    x = table[token_ids.long()].to(torch.float32)
+    if position_table is not None:
+        x = x + position_table[positions.long()].to(torch.float32)
+    return x
 
 
 def add_rmsnorm(residual, delta, weight, eps, unit_offset, out_dtype):
@@ -322,7 +325,7 @@ def qkv_prepare(qkv, n_heads, n_kv, head_dim, value_dim, positions, act_dtype, q
 
 
 def attention_masked(q, n_heads, n_kv, head_dim, value_dim, k_cache, v_cache, page_size, scale, ctx, group, window=0,
-                     keep_first=0, softcap=0.0, value_rotation=None, gate=None, gate_col=0):
+                     keep_first=0, softcap=0.0, value_rotation=None, gate=None, gate_col=0, gate_elems=1, distance_bias=None):
     n = q.shape[0]
     positions, token_seq = ctx.arrays["positions"], ctx.arrays["token_seq"]
     bt = ctx.arrays[f"block_table_g{group}"]
@@ -343,18 +346,22 @@ def attention_masked(q, n_heads, n_kv, head_dim, value_dim, k_cache, v_cache, pa
             s = (k[:, g, :] @ qh[t, h]) * scale
             if softcap:
                 s = softcap * torch.tanh(s / softcap)
+            if distance_bias is not None:
+                s = s + distance_bias[(pos - j).clamp(max=distance_bias.shape[0] - 1).long(), h]
             out[t, h] = torch.softmax(s, dim=0) @ v[:, g, :]
-    out = attention_finish(out, positions, n_heads, value_dim, value_rotation, gate, gate_col)
+    out = attention_finish(out, positions, n_heads, value_dim, value_rotation, gate, gate_col, gate_elems)
     return out.reshape(n, n_heads * value_dim).to(q.dtype)
 
 
-def attention_finish(out, positions, n_heads, value_dim, value_rotation=None, gate=None, gate_col=0):
+def attention_finish(out, positions, n_heads, value_dim, value_rotation=None, gate=None, gate_col=0, gate_elems=1):
     shape = out.shape
     o = out.reshape(out.shape[0], n_heads, value_dim).to(torch.float32)
     if value_rotation is not None:
         pos = positions.long()
         o = _turn(o, value_rotation.cos[pos][:, None, :], value_rotation.sin[pos][:, None, :], value_dim, value_rotation.interleaved, -1.0)
-    if gate is not None:
+    if gate is not None and gate_elems > 1:
+        o = o * torch.sigmoid(gate[:, gate_col: gate_col + n_heads * value_dim].to(torch.float32)).view(-1, n_heads, value_dim)
+    elif gate is not None:
         o = o * torch.sigmoid(gate[:, gate_col: gate_col + n_heads].to(torch.float32))[:, :, None]
     return o.reshape(shape).to(out.dtype)
 
@@ -406,15 +413,18 @@ def rglru(u, y, x, wa_t, ba, wi_t, bi, lam, rate, s_state, conv_state, taps, ctx
 
 
 def moe_experts(x, token_ids, table, w_gate_up, w_down, activation):
-    n, hidden = x.shape
+    """``token_ids`` None: ``table`` has a row per token and ``x`` a row per (token, choice)."""
     top = table.shape[1]
+    hidden = x.shape[1]
+    n = x.shape[0] if token_ids is not None else table.shape[0]
     rows = torch.empty((n * top, hidden), dtype=torch.float32, device=x.device)
     xf = x.to(torch.float32)
     for t in range(n):
         for k in range(top):
-            e = int(table[int(token_ids[t]), k])
-            g = w_gate_up[e, 0].to(torch.float32) @ xf[t]
-            u = w_gate_up[e, 1].to(torch.float32) @ xf[t]
+            e = int(table[int(token_ids[t]) if token_ids is not None else t, k])
+            xin = xf[t] if token_ids is not None else xf[t * top + k]
+            g = w_gate_up[e, 0].to(torch.float32) @ xin
+            u = w_gate_up[e, 1].to(torch.float32) @ xin
             yv = gated_pair(g, u, activation).to(x.dtype).to(torch.float32)
             rows[t * top + k] = w_down[e].to(torch.float32) @ yv
     return rows
@@ -484,8 +494,11 @@ def latent_prepare(proj, q_rank, q_norm, eps, act_dtype, kv_col=0, kv_rank=0, ro
     if kv_rank:
         c = _rmsnorm(p[:, kv_col: kv_col + kv_rank], kv_norm, eps, False)
         pos = positions.long()
-        r = _turn(p[:, kv_col + kv_rank: kv_col + kv_rank + rot_dim], rotation.cos[pos], rotation.sin[pos], rot_dim, rotation.interleaved)
-        row = torch.cat([c, r], dim=1).to(pages.dtype)
+        row = c
+        if rot_dim:
+            r = _turn(p[:, kv_col + kv_rank: kv_col + kv_rank + rot_dim], rotation.cos[pos], rotation.sin[pos], rot_dim, rotation.interleaved)
+            row = torch.cat([c, r], dim=1)
+        row = row.to(pages.dtype)
         s = slots.long()
         pages[s // page_size, 0, s % page_size, :] = row
         if values is not None:  # the latent once more, transposed
@@ -493,7 +506,8 @@ def latent_prepare(proj, q_rank, q_norm, eps, act_dtype, kv_col=0, kv_rank=0, ro
     return c_q
 
 
-def head_linear(x, w, n_heads, in_dim, out_dim, out_dtype, tail=0, rotation=None, positions=None, gate=None, gate_col=0, w_t=None):
+def head_linear(x, w, n_heads, in_dim, out_dim, out_dtype, tail=0, rotation=None, positions=None, gate=None, gate_col=0, w_t=None,
+                gate_elems=1):
     """Per head, out[n, h, :out_dim] = x[n, h, :in_dim] . w[h] (w [heads, in, out]); ``tail`` more elements of
     every head of x follow the product, turned by the token's position; ``gate``: the head's output times
     the sigmoid of column gate_col + h of ``gate``."""
@@ -504,12 +518,14 @@ def head_linear(x, w, n_heads, in_dim, out_dim, out_dtype, tail=0, rotation=None
         pos = positions.long()
         t = _turn(xh[..., in_dim:], rotation.cos[pos][:, None, :], rotation.sin[pos][:, None, :], tail, rotation.interleaved)
         out = torch.cat([out, t], dim=-1)
-    if gate is not None:
+    if gate is not None and gate_elems > 1:
+        out = out * torch.sigmoid(gate[:, gate_col: gate_col + n_heads * out_dim].float()).view(n, n_heads, out_dim)
+    elif gate is not None:
         out = out * torch.sigmoid(gate[:, gate_col: gate_col + n_heads].float())[:, :, None]
     return out.reshape(n, -1).to(out_dtype)
 
 
-def latent_attention(q_lat, pages, n_heads, kv_rank, rot_dim, scale, ctx, group, page_size, tiles=None, values=None):
+def latent_attention(q_lat, pages, n_heads, kv_rank, rot_dim, scale, ctx, group, page_size, tiles=None, values=None, sink=None):
     a = ctx.arrays
     n = q_lat.shape[0]
     width = kv_rank + rot_dim
@@ -520,7 +536,10 @@ def latent_attention(q_lat, pages, n_heads, kv_rank, rot_dim, scale, ctx, group,
         seq, p = int(a["token_seq"][t]), int(a["positions"][t])
         idx = torch.arange(p + 1)
         rows = pages[bt[seq, idx // page_size].long(), 0, idx % page_size, :].float()
-        prob = torch.softmax((q[t] @ rows.T) * scale, dim=-1)
+        scores = (q[t] @ rows.T) * scale
+        if sink is not None:  # a score with no key and no value
+            scores = torch.cat([scores, sink.float()[:, None]], dim=1)
+        prob = torch.softmax(scores, dim=-1)[:, : rows.shape[0]]
         out[t] = prob @ rows[:, :kv_rank]
     return out.view(n, n_heads * kv_rank)
 
@@ -539,25 +558,29 @@ def conv_state_push(x, state, ctx):
         state[slot] = torch.cat([state[slot], x[q0: q0 + ql].to(state.dtype)], dim=0)[-keep:]
 
 
-def linear_state_scan(qkv, n_heads, n_kv, dim, vdim, state, ctx, q_scale=1.0, unit_eps=None, decay=None, beta=None):
+def linear_state_scan(qkv, n_heads, n_kv, dim, vdim, state, ctx, q_scale=1.0, unit_eps=None, decay=None, beta=None, columns=None,
+                      skip=None):
     a = ctx.arrays
     n = qkv.shape[0]
     x = qkv.float()
     kd = n_kv * dim
-    q, k, v = x[:, :kd].reshape(n, n_kv, dim), x[:, kd: 2 * kd].reshape(n, n_kv, dim), x[:, 2 * kd: 2 * kd + n_heads * vdim].reshape(n, n_heads, vdim)
+    qc, kc, vc = columns if columns is not None else (0, kd, 2 * kd)
+    q, k, v = x[:, qc: qc + kd].reshape(n, n_kv, dim), x[:, kc: kc + kd].reshape(n, n_kv, dim), x[:, vc: vc + n_heads * vdim].reshape(n, n_heads, vdim)
     if unit_eps is not None:
         q = q / torch.sqrt((q * q).sum(-1, keepdim=True) + unit_eps)
         k = k / torch.sqrt((k * k).sum(-1, keepdim=True) + unit_eps)
     q = q * q_scale
     if decay[0] == "head":
         _, src, col, a_log, dt_bias = decay
-        g = torch.exp(-torch.exp(a_log.float()) * torch.nn.functional.softplus(src[:, col: col + n_heads].float() + dt_bias.float()))
+        step = torch.nn.functional.softplus(src[:, col: col + n_heads].float() + dt_bias.float())
+        g = torch.exp(-torch.exp(a_log.float()) * step)
         g = g[:, :, None].expand(n, n_heads, dim)
     else:
         _, src, col, bias, tau = decay
         z = src[:, col: col + n_heads * dim].float() + bias.float()
         g = torch.exp(torch.nn.functional.logsigmoid(z) / tau).view(n, n_heads, dim)
-    b = None if beta is None else torch.sigmoid(beta[0][:, beta[1]: beta[1] + n_heads].float())
+    by_step = isinstance(beta, str)  # "step": u = dt v, no delta rule
+    b = None if beta is None or by_step else torch.sigmoid(beta[0][:, beta[1]: beta[1] + n_heads].float())
     out = torch.empty((n, n_heads, vdim), dtype=torch.float32, device=qkv.device)
     per = n_heads // n_kv
     for s in range(a["seq_qstart"].numel()):
@@ -568,18 +591,46 @@ def linear_state_scan(qkv, n_heads, n_kv, dim, vdim, state, ctx, q_scale=1.0, un
                 kk, qq = k[t, h // per], q[t, h // per]
                 Sh = g[t, h][:, None] * S[h]
                 u = v[t, h] if b is None else b[t, h] * (v[t, h] - Sh.T @ kk)
+                if by_step:
+                    u = step[t, h] * v[t, h]
                 Sh = Sh + torch.outer(kk, u)
                 out[t, h] = Sh.T @ qq
+                if skip is not None:
+                    out[t, h] += skip[h].float() * v[t, h]
                 S[h] = Sh
         state[slot] = S
     return out.view(n, n_heads * vdim)
 
 
-def gated_head_norm(o, weight, eps, gate, gate_col, n_heads, vdim, out_dtype):
+def gated_head_norm(o, weight, eps, gate, gate_col, n_heads, vdim, out_dtype, gate_first=False):
     n = o.shape[0]
-    y = _rmsnorm(o.float().view(n, n_heads, vdim), weight, eps, False).reshape(n, -1)
     g = gate[:, gate_col: gate_col + n_heads * vdim].float()
+    w = weight.float() if weight.numel() == vdim else weight.float().view(n_heads, vdim)
+    if gate_first:
+        return _rmsnorm((o.float() * g * torch.sigmoid(g)).view(n, n_heads, vdim), w, eps, False).reshape(n, -1).to(out_dtype)
+    y = _rmsnorm(o.float().view(n, n_heads, vdim), w, eps, False).reshape(n, -1)
     return (y * g * torch.sigmoid(g)).to(out_dtype)
+
+
+def moe_router_topk(logits, x, top, experts=None):
+    experts = logits.shape[1] if experts is None else experts
+    z = logits[:, :experts].float()
+    n = z.shape[0]
+    choice = torch.empty((n, top), dtype=torch.int32, device=x.device)
+    xs = torch.empty((n * top, x.shape[1]), dtype=x.dtype, device=x.device)
+    for t in range(n):
+        left = z[t].clone()
+        for k in range(top):
+            e = int(torch.argmax(left))  # (the first of equals)
+            choice[t, k] = e
+            xs[t * top + k] = (x[t].float() * torch.sigmoid(z[t, e])).to(x.dtype)
+            left[e] = -math.inf
+    return choice, xs
+
+
+def moe_combine(dense, rows, top, weight=1.0):
+    out = rows.view(rows.shape[0] // top, top, rows.shape[1]).sum(1) * weight
+    return out if dense is None else out + dense.float()
 
 
 RefOps.sandwich_norm = staticmethod(sandwich_norm)
@@ -594,3 +645,6 @@ RefOps.causal_conv = staticmethod(causal_conv_act)
 RefOps.conv_state_push = staticmethod(conv_state_push)
 RefOps.linear_state_scan = staticmethod(linear_state_scan)
 RefOps.gated_head_norm = staticmethod(gated_head_norm)
+RefOps.moe_router_topk = staticmethod(moe_router_topk)
+RefOps.moe_combine = staticmethod(moe_combine)
+RefOps.moe_experts = staticmethod(moe_experts)

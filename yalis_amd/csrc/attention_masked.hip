@@ -375,7 +375,8 @@ __global__ __launch_bounds__(64) void attn_masked_kernel(
     const int32_t* __restrict__ block_table, int table_width, int page_size, int head_dim, int v_dim, int n_heads,
     int n_kv, float scale, float softcap, int window, int keep_first, int tiled, const float* __restrict__ v_cos,
     const float* __restrict__ v_sin, int v_interleaved, int v_max_pos, const TG* __restrict__ gate_src,
-    int gate_splits, size_t gate_split_stride, int gate_round, int gate_stride, int gate_col0) {
+    int gate_splits, size_t gate_split_stride, int gate_round, int gate_stride, int gate_col0, int gate_elems,
+    const float* __restrict__ dist_bias, int bias_rows) {
   const size_t slab_k = static_cast<size_t>(page_size) * head_dim, slab_v = static_cast<size_t>(page_size) * v_dim;
   __shared__ float qs[kMaxHead];
   __shared__ float os[kMaxHead];
@@ -410,6 +411,8 @@ __global__ __launch_bounds__(64) void attn_masked_kernel(
         dot = fmaf(qs[d], to_f32<T>(kp[cache_k_offset(tiled, page_size, head_dim, off, d)]), dot);
       s = dot * scale;
       if (softcap > 0.f) s = softcap * tanhf(s / softcap);
+      // a learned number per (distance, head), added to the scaled score as it is
+      if (dist_bias != nullptr) s += dist_bias[static_cast<size_t>(min(pos - key, bias_rows - 1)) * n_heads + h];
     }
     const float m_new = fmaxf(m, wave_max(s));  // finite: the tile holds at least one key
     const float p = valid ? expf(s - m_new) : 0.f;
@@ -443,8 +446,8 @@ __global__ __launch_bounds__(64) void attn_masked_kernel(
   }
   __syncthreads();
   float gate = 1.f;
-  if (gate_src != nullptr)
-    gate = head_gate<TG>(gate_src, gate_splits, gate_split_stride, gate_round, static_cast<size_t>(n) * gate_stride + gate_col0 + h);
+  const size_t gate_at = static_cast<size_t>(n) * gate_stride + gate_col0 + static_cast<size_t>(h) * gate_elems;
+  if (gate_src != nullptr && gate_elems == 1) gate = head_gate<TG>(gate_src, gate_splits, gate_split_stride, gate_round, gate_at);
   const float *cr = nullptr, *sr = nullptr;
   if (v_cos != nullptr) {
     const int p = min(pos, v_max_pos - 1);
@@ -457,18 +460,25 @@ __global__ __launch_bounds__(64) void attn_masked_kernel(
     const int d = lane + 64 * i;
     if (d < v_dim) {
       const float v = cr != nullptr ? rotated_element(os, d, v_dim, v_interleaved, cr, sr, -1.f) : os[d];
+      if (gate_src != nullptr && gate_elems > 1) gate = head_gate<TG>(gate_src, gate_splits, gate_split_stride, gate_round, gate_at + d);
       orow[d] = from_f32<T>(v * gate);
     }
   }
 }
 
+// gate_elems: 1, a gate per head in column gate_col0 + h, or v_dim, one per output element in column gate_col0 + h *
+// v_dim + d.  dist_bias [bias_rows][n_heads] float32 or null: what is added to the score of a key at distance n (the
+// last row for every larger distance).
 extern "C" int yk_attn_masked(const void* q, int q_stride, void* out, const void* k_cache, const void* v_cache, int dtype,
                               const int32_t* positions, const int32_t* token_seq, const int32_t* block_table,
                               int table_width, int n_tokens, int page_size, int head_dim, int v_dim, int n_heads, int n_kv,
                               float scale, float softcap, int window, int keep_first, int tiled, const float* v_cos,
                               const float* v_sin, int v_interleaved, int v_max_pos, const void* gate_src, int gate_dtype,
-                              int gate_splits, int gate_round, int gate_stride, int gate_col0, hipStream_t stream) {
+                              int gate_splits, int gate_round, int gate_stride, int gate_col0, int gate_elems,
+                              const float* dist_bias, int bias_rows, hipStream_t stream) {
   YK_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0, "attn_masked: bad head counts");
+  YK_REQUIRE(gate_src == nullptr || gate_elems == 1 || gate_elems == v_dim, "attn_masked: a gate per head or per output element");
+  YK_REQUIRE(dist_bias == nullptr || bias_rows >= 1, "attn_masked: an empty table of biases");
   YK_REQUIRE(head_dim > 0 && head_dim <= kMaxHead && v_dim > 0 && v_dim <= kMaxHead, "attn_masked: heads of 1 to 256 elements");
   YK_REQUIRE(page_size > 0 && table_width > 0, "attn_masked: bad page table");
   YK_REQUIRE(window >= 0 && keep_first >= 0 && softcap >= 0.f, "attn_masked: window, keep_first and softcap must not be negative");
@@ -485,7 +495,8 @@ extern "C" int yk_attn_masked(const void* q, int q_stride, void* out, const void
         static_cast<const T*>(q), q_stride, static_cast<T*>(out), static_cast<const T*>(k_cache),              \
         static_cast<const T*>(v_cache), positions, token_seq, block_table, table_width, page_size, head_dim,   \
         v_dim, n_heads, n_kv, scale, softcap, window, keep_first, tiled, v_cos, v_sin, v_interleaved, v_max_pos, \
-        static_cast<const TG*>(gate_src), gate_splits, gstride, gate_round, gate_stride, gate_col0);           \
+        static_cast<const TG*>(gate_src), gate_splits, gstride, gate_round, gate_stride, gate_col0, gate_elems, \
+        dist_bias, bias_rows);                                                                                 \
     return yk_check_launch("attn_masked");                                                                     \
   }
   YK_CASE(YK_F32, float, YK_F32, float)
@@ -499,15 +510,15 @@ template <typename T, typename TG>
 __global__ __launch_bounds__(64) void attn_finish_kernel(
     T* __restrict__ out, const int32_t* __restrict__ positions, int v_dim, int n_heads, const float* __restrict__ v_cos,
     const float* __restrict__ v_sin, int v_interleaved, int v_max_pos, const TG* __restrict__ gate_src, int gate_splits,
-    size_t gate_split_stride, int gate_round, int gate_stride, int gate_col0) {
+    size_t gate_split_stride, int gate_round, int gate_stride, int gate_col0, int gate_elems) {
   __shared__ float os[kMaxHead];
   const int n = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   T* orow = out + (static_cast<size_t>(n) * n_heads + h) * v_dim;
   for (int d = lane; d < v_dim; d += 64) os[d] = to_f32<T>(orow[d]);
   __syncthreads();
   float gate = 1.f;
-  if (gate_src != nullptr)
-    gate = head_gate<TG>(gate_src, gate_splits, gate_split_stride, gate_round, static_cast<size_t>(n) * gate_stride + gate_col0 + h);
+  const size_t gate_at = static_cast<size_t>(n) * gate_stride + gate_col0 + static_cast<size_t>(h) * gate_elems;
+  if (gate_src != nullptr && gate_elems == 1) gate = head_gate<TG>(gate_src, gate_splits, gate_split_stride, gate_round, gate_at);
   const float *cr = nullptr, *sr = nullptr;
   if (v_cos != nullptr) {
     const int p = min(positions[n], v_max_pos - 1);
@@ -516,6 +527,7 @@ __global__ __launch_bounds__(64) void attn_finish_kernel(
   }
   for (int d = lane; d < v_dim; d += 64) {
     const float v = cr != nullptr ? rotated_element(os, d, v_dim, v_interleaved, cr, sr, -1.f) : os[d];
+    if (gate_src != nullptr && gate_elems > 1) gate = head_gate<TG>(gate_src, gate_splits, gate_split_stride, gate_round, gate_at + d);
     orow[d] = from_f32<T>(v * gate);
   }
 }
@@ -523,8 +535,9 @@ __global__ __launch_bounds__(64) void attn_finish_kernel(
 extern "C" int yk_attn_finish(void* out, int dtype, const int32_t* positions, int n_tokens, int v_dim, int n_heads,
                               const float* v_cos, const float* v_sin, int v_interleaved, int v_max_pos,
                               const void* gate_src, int gate_dtype, int gate_splits, int gate_round, int gate_stride,
-                              int gate_col0, hipStream_t stream) {
+                              int gate_col0, int gate_elems, hipStream_t stream) {
   YK_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_heads <= 65535 && v_dim > 0 && v_dim <= kMaxHead, "attn_finish: bad sizes");
+  YK_REQUIRE(gate_src == nullptr || gate_elems == 1 || gate_elems == v_dim, "attn_finish: a gate per head or per output element");
   YK_REQUIRE(v_cos == nullptr || (v_sin != nullptr && v_max_pos > 0 && v_dim % 2 == 0), "attn_finish: value tables need an even value_dim");
   if (n_tokens == 0 || (v_cos == nullptr && gate_src == nullptr)) return 0;
   dim3 grid(n_tokens, n_heads), block(64);
@@ -533,7 +546,8 @@ extern "C" int yk_attn_finish(void* out, int dtype, const int32_t* positions, in
   if (dtype == D && (gate_src == nullptr ? GD == D : gate_dtype == GD)) {                               \
     attn_finish_kernel<T, TG><<<grid, block, 0, stream>>>(static_cast<T*>(out), positions, v_dim, n_heads, v_cos, v_sin, \
                                                           v_interleaved, v_max_pos, static_cast<const TG*>(gate_src),   \
-                                                          gate_splits, gstride, gate_round, gate_stride, gate_col0);    \
+                                                          gate_splits, gstride, gate_round, gate_stride, gate_col0,     \
+                                                          gate_elems);                                                  \
     return yk_check_launch("attn_finish");                                                              \
   }
   YK_CASE(YK_F32, float, YK_F32, float)

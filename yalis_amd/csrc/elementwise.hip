@@ -14,22 +14,43 @@
 extern "C" int yk_cache_tiled(int dtype, int head_dim, int page_size) { return cache_is_tiled(dtype, head_dim, page_size) ? 1 : 0; }
 
 // ------------------------------------------------------------------------- embedding
-// out[n, :] = float(table[ids[n], :])
+// out[n, :] = float(table[ids[n], :]) (+ float(pos_table[positions[n], :]): a learned vector per
+// absolute position, added in float32)
 template <typename T>
 __global__ void embed_kernel(const int32_t* __restrict__ ids, const T* __restrict__ table,
-                             float* __restrict__ out, int width, int vocab) {
+                             float* __restrict__ out, int width, int vocab, const int32_t* __restrict__ positions,
+                             const T* __restrict__ pos_table, int pos_rows) {
   const int n = blockIdx.x;
   int id = ids[n];
   // ids are checked on the host; clamp so that a bad id cannot read out of bounds
   id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
   const T* src = table + static_cast<size_t>(id) * width;
   float* dst = out + static_cast<size_t>(n) * width;
+  if (pos_table != nullptr) {
+    int p = positions[n];
+    p = p < 0 ? 0 : (p >= pos_rows ? pos_rows - 1 : p);
+    const T* ps = pos_table + static_cast<size_t>(p) * width;
+    for (int c = threadIdx.x; c < width; c += blockDim.x) dst[c] = to_f32<T>(src[c]) + to_f32<T>(ps[c]);
+    return;
+  }
   for (int c = threadIdx.x; c < width; c += blockDim.x) dst[c] = to_f32<T>(src[c]);
+}
+
+__device__ __forceinline__ void embed_unpack8(const uint4 raw, float4& lo, float4& hi) {
+  lo.x = __uint_as_float(raw.x << 16);
+  lo.y = __uint_as_float(raw.x & 0xffff0000u);
+  lo.z = __uint_as_float(raw.y << 16);
+  lo.w = __uint_as_float(raw.y & 0xffff0000u);
+  hi.x = __uint_as_float(raw.z << 16);
+  hi.y = __uint_as_float(raw.z & 0xffff0000u);
+  hi.z = __uint_as_float(raw.w << 16);
+  hi.w = __uint_as_float(raw.w & 0xffff0000u);
 }
 
 // eight elements per thread, no loop (bfloat16 tables whose width is a multiple of 8)
 __global__ void embed_bf16x8_kernel(const int32_t* __restrict__ ids, const bf16_t* __restrict__ table,
-                                    float* __restrict__ out, int width, int vocab, size_t total_vec) {
+                                    float* __restrict__ out, int width, int vocab, size_t total_vec,
+                                    const int32_t* __restrict__ positions, const bf16_t* __restrict__ pos_table, int pos_rows) {
   const size_t v = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x;
   if (v >= total_vec) return;
   const int per_row = width / 8;
@@ -37,38 +58,43 @@ __global__ void embed_bf16x8_kernel(const int32_t* __restrict__ ids, const bf16_
   const int c = static_cast<int>(v % per_row) * 8;
   int id = ids[n];
   id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
-  const uint4 raw = *reinterpret_cast<const uint4*>(table + static_cast<size_t>(id) * width + c);
-  const uint32_t wds[4] = {raw.x, raw.y, raw.z, raw.w};
   float4 lo, hi;
-  lo.x = __uint_as_float(wds[0] << 16);
-  lo.y = __uint_as_float(wds[0] & 0xffff0000u);
-  lo.z = __uint_as_float(wds[1] << 16);
-  lo.w = __uint_as_float(wds[1] & 0xffff0000u);
-  hi.x = __uint_as_float(wds[2] << 16);
-  hi.y = __uint_as_float(wds[2] & 0xffff0000u);
-  hi.z = __uint_as_float(wds[3] << 16);
-  hi.w = __uint_as_float(wds[3] & 0xffff0000u);
+  embed_unpack8(*reinterpret_cast<const uint4*>(table + static_cast<size_t>(id) * width + c), lo, hi);
+  if (pos_table != nullptr) {
+    int p = positions[n];
+    p = p < 0 ? 0 : (p >= pos_rows ? pos_rows - 1 : p);
+    float4 plo, phi;
+    embed_unpack8(*reinterpret_cast<const uint4*>(pos_table + static_cast<size_t>(p) * width + c), plo, phi);
+    lo.x += plo.x; lo.y += plo.y; lo.z += plo.z; lo.w += plo.w;
+    hi.x += phi.x; hi.y += phi.y; hi.z += phi.z; hi.w += phi.w;
+  }
   float* dst = out + n * width + c;
   *reinterpret_cast<float4*>(dst) = lo;
   *reinterpret_cast<float4*>(dst + 4) = hi;
 }
 
+// positions / pos_table (of the table's dtype, pos_rows rows) null: the token's row alone
 extern "C" int yk_embed(const int32_t* ids, const void* table, int table_dtype, float* out,
-                        int n_tokens, int width, int vocab, hipStream_t stream) {
+                        int n_tokens, int width, int vocab, const int32_t* positions, const void* pos_table, int pos_rows,
+                        hipStream_t stream) {
   YK_REQUIRE(n_tokens >= 0 && width > 0 && vocab > 0, "embed: bad sizes");
+  YK_REQUIRE(pos_table == nullptr || (positions != nullptr && pos_rows > 0), "embed: a position table needs positions");
   if (n_tokens == 0) return 0;
   if (table_dtype == YK_BF16 && width % 8 == 0 && reinterpret_cast<uintptr_t>(table) % 16 == 0 &&
-      reinterpret_cast<uintptr_t>(out) % 16 == 0) {
+      reinterpret_cast<uintptr_t>(out) % 16 == 0 && reinterpret_cast<uintptr_t>(pos_table) % 16 == 0) {
     const size_t total_vec = static_cast<size_t>(n_tokens) * (width / 8);
     embed_bf16x8_kernel<<<static_cast<unsigned>((total_vec + 255) / 256), 256, 0, stream>>>(
-        ids, static_cast<const bf16_t*>(table), out, width, vocab, total_vec);
+        ids, static_cast<const bf16_t*>(table), out, width, vocab, total_vec, positions, static_cast<const bf16_t*>(pos_table),
+        pos_rows);
     return yk_check_launch("embed");
   }
   dim3 grid(n_tokens), block(256);
   if (table_dtype == YK_F32)
-    embed_kernel<float><<<grid, block, 0, stream>>>(ids, static_cast<const float*>(table), out, width, vocab);
+    embed_kernel<float><<<grid, block, 0, stream>>>(ids, static_cast<const float*>(table), out, width, vocab, positions,
+                                                    static_cast<const float*>(pos_table), pos_rows);
   else if (table_dtype == YK_BF16)
-    embed_kernel<bf16_t><<<grid, block, 0, stream>>>(ids, static_cast<const bf16_t*>(table), out, width, vocab);
+    embed_kernel<bf16_t><<<grid, block, 0, stream>>>(ids, static_cast<const bf16_t*>(table), out, width, vocab, positions,
+                                                     static_cast<const bf16_t*>(pos_table), pos_rows);
   else
     return yk_fail("embed: unsupported table dtype");
   return yk_check_launch("embed");

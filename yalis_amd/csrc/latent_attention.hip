@@ -109,7 +109,7 @@ __global__ __launch_bounds__(kHeadOut * kHeadSlices) void head_linear_kernel(
     const TX* __restrict__ x, int x_stride, const TW* __restrict__ w, TO* __restrict__ out, int out_stride, int in_dim,
     int out_dim, int tail, const int32_t* __restrict__ positions, const float* __restrict__ cos_t,
     const float* __restrict__ sin_t, int interleaved, const TG* __restrict__ gate, int gate_stride, int gate_col,
-    int n_tokens) {
+    int gate_elems, int n_tokens) {
   extern __shared__ float xs[];  // [kHeadTokens][in_dim + tail], then [kHeadSlices][kHeadTokens][kHeadOut]
   const int n0 = blockIdx.x * kHeadTokens, h = blockIdx.y, o0 = blockIdx.z * kHeadOut;
   const int count = min(kHeadTokens, n_tokens - n0);
@@ -151,7 +151,9 @@ __global__ __launch_bounds__(kHeadOut * kHeadSlices) void head_linear_kernel(
     float v = 0.f;
 #pragma unroll
     for (int sl = 0; sl < kHeadSlices; ++sl) v += part[(sl * kHeadTokens + t) * kHeadOut + oc];
-    if (gate != nullptr) v *= 1.f / (1.f + expf(-to_f32<TG>(gate[static_cast<size_t>(n0 + t) * gate_stride + gate_col + h])));
+    if (gate != nullptr)
+      v *= 1.f / (1.f + expf(-to_f32<TG>(gate[static_cast<size_t>(n0 + t) * gate_stride + gate_col + h * gate_elems +
+                                                  (gate_elems > 1 ? o0 + oc : 0)])));
     out[static_cast<size_t>(n0 + t) * out_stride + h * ow + o0 + oc] = from_f32<TO>(v);
   }
   if (blockIdx.z != 0) return;
@@ -173,8 +175,9 @@ __global__ __launch_bounds__(kHeadOut * kHeadSlices) void head_linear_kernel(
 extern "C" int yk_head_linear(const void* x, int x_stride, int x_dtype, const void* w, int w_dtype, void* out, int out_dtype,
                               int n_heads, int in_dim, int out_dim, int tail, const int32_t* positions, const float* cos_t,
                               const float* sin_t, int interleaved, const void* gate, int gate_dtype, int gate_stride,
-                              int gate_col, int n_tokens, hipStream_t stream) {
+                              int gate_col, int gate_elems, int n_tokens, hipStream_t stream) {
   YK_REQUIRE(n_tokens >= 0 && n_heads > 0 && in_dim > 0 && out_dim > 0 && tail >= 0 && tail % 2 == 0, "head_linear: bad sizes");
+  YK_REQUIRE(gate == nullptr || gate_elems == 1 || gate_elems == out_dim, "head_linear: a gate per head or per output element");
   YK_REQUIRE(x_stride >= n_heads * (in_dim + tail), "head_linear: the input's rows are shorter than its heads");
   YK_REQUIRE(tail == 0 || (positions != nullptr && cos_t != nullptr && sin_t != nullptr), "head_linear: a turned tail needs positions and tables");
   const int slices = 4;
@@ -190,12 +193,12 @@ extern "C" int yk_head_linear(const void* x, int x_stride, int x_dtype, const vo
       head_linear_kernel<TX, TW, TG, TO, 1><<<grid, kHeadOut, lds, stream>>>(                                        \
           static_cast<const TX*>(x), x_stride, static_cast<const TW*>(w), static_cast<TO*>(out), out_stride, in_dim, \
           out_dim, tail, positions, cos_t, sin_t, interleaved, static_cast<const TG*>(gate), gate_stride, gate_col,  \
-          n_tokens);                                                                                                 \
+          gate_elems, n_tokens);                                                                                              \
     else                                                                                                             \
       head_linear_kernel<TX, TW, TG, TO, 4><<<grid, kHeadOut * 4, lds, stream>>>(                                    \
           static_cast<const TX*>(x), x_stride, static_cast<const TW*>(w), static_cast<TO*>(out), out_stride, in_dim, \
           out_dim, tail, positions, cos_t, sin_t, interleaved, static_cast<const TG*>(gate), gate_stride, gate_col,  \
-          n_tokens);                                                                                                 \
+          gate_elems, n_tokens);                                                                                              \
     return yk_check_launch("head_linear");                                                                           \
   }
   YK_CASE(YK_F32, float, YK_F32, float, YK_F32, float, YK_F32, float)
@@ -252,7 +255,7 @@ __global__ __launch_bounds__(256) void head_linear_mfma_kernel(
     const TX* __restrict__ x, int x_stride, const bf16_t* __restrict__ w_t, TO* __restrict__ out, int out_stride, int in_dim,
     int out_dim, int tail, const int32_t* __restrict__ positions, const float* __restrict__ cos_t,
     const float* __restrict__ sin_t, int interleaved, const TG* __restrict__ gate, int gate_stride, int gate_col,
-    int n_tokens) {
+    int gate_elems, int n_tokens) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x % kWave;
   const int r = lane % 16, g = lane / 16;
   const int n0 = (blockIdx.x * 4 + wave) * 16, h = blockIdx.y, o0 = blockIdx.z * 64;
@@ -285,10 +288,14 @@ __global__ __launch_bounds__(256) void head_linear_mfma_kernel(
     const int n = n0 + 4 * g + i;
     if (n >= n_tokens) continue;
     float gv = 1.f;
-    if (gate != nullptr) gv = 1.f / (1.f + expf(-to_f32<TG>(gate[static_cast<size_t>(n) * gate_stride + gate_col + h])));
+    const TG* grow = gate == nullptr ? nullptr : gate + static_cast<size_t>(n) * gate_stride + gate_col + h * gate_elems;
+    if (gate != nullptr && gate_elems == 1) gv = 1.f / (1.f + expf(-to_f32<TG>(grow[0])));
 #pragma unroll
     for (int j = 0; j < 4; ++j)
-      if (j < n_tiles) out[static_cast<size_t>(n) * out_stride + h * ow + o0 + 16 * j + r] = from_f32<TO>(acc[j][i] * gv);
+      if (j < n_tiles) {
+        if (gate != nullptr && gate_elems > 1) gv = 1.f / (1.f + expf(-to_f32<TG>(grow[o0 + 16 * j + r])));
+        out[static_cast<size_t>(n) * out_stride + h * ow + o0 + 16 * j + r] = from_f32<TO>(acc[j][i] * gv);
+      }
   }
   if (blockIdx.z != 0 || tail == 0) return;
   const int half = tail / 2;
@@ -312,7 +319,8 @@ extern "C" int yk_head_linear_mfma_ok(int in_dim, int out_dim, int tail) { retur
 extern "C" int yk_head_linear_mfma(const void* x, int x_stride, int x_dtype, const void* w_t, void* out, int out_dtype, int n_heads,
                                    int in_dim, int out_dim, int tail, const int32_t* positions, const float* cos_t,
                                    const float* sin_t, int interleaved, const void* gate, int gate_dtype, int gate_stride,
-                                   int gate_col, int n_tokens, hipStream_t stream) {
+                                   int gate_col, int gate_elems, int n_tokens, hipStream_t stream) {
+  YK_REQUIRE(gate == nullptr || gate_elems == 1 || gate_elems == out_dim, "head_linear_mfma: a gate per head or per output element");
   YK_REQUIRE(n_tokens >= 0 && n_heads > 0 && yk_head_linear_mfma_ok(in_dim, out_dim, tail), "head_linear_mfma: sizes it is not built for");
   YK_REQUIRE(x_stride >= n_heads * (in_dim + tail) && x_stride % 8 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 &&
                  reinterpret_cast<uintptr_t>(w_t) % 16 == 0,
@@ -327,7 +335,7 @@ extern "C" int yk_head_linear_mfma(const void* x, int x_stride, int x_dtype, con
     head_linear_mfma_kernel<TX, TG, TO><<<grid, 256, 0, stream>>>(                                                      \
         static_cast<const TX*>(x), x_stride, static_cast<const bf16_t*>(w_t), static_cast<TO*>(out), out_stride, in_dim, \
         out_dim, tail, positions, cos_t, sin_t, interleaved, static_cast<const TG*>(gate), gate_stride, gate_col,       \
-        n_tokens);                                                                                                      \
+        gate_elems, n_tokens);                                                                                                      \
     return yk_check_launch("head_linear_mfma");                                                                         \
   }
   YK_CASE(YK_BF16, bf16_t, YK_F32, float, YK_F32, float)
@@ -349,7 +357,7 @@ template <typename T, int RPL>
 __global__ __launch_bounds__(64 * kLatWaves) void latent_attention_kernel(
     const float* __restrict__ q_lat, const T* __restrict__ pages, const int32_t* __restrict__ tiles,
     const int32_t* __restrict__ block_table, int table_width, int page_size, int n_heads, int heads_per_group, int kv_rank,
-    int rot_dim, float scale, int KB, int pad, float* __restrict__ out) {
+    int rot_dim, float scale, int KB, int pad, const float* __restrict__ sink, float* __restrict__ out) {
   extern __shared__ unsigned char lds_raw[];
   const int width = kv_rank + rot_dim, row_w = width + pad;
   T* kblock = reinterpret_cast<T*>(lds_raw);                                             // [KB][row_w]
@@ -375,8 +383,9 @@ __global__ __launch_bounds__(64 * kLatWaves) void latent_attention_kernel(
     tok[it] = tok0 + (live[it] ? t : 0);
     if (!live[it]) head[it] = 0;
     pos[it] = pos0 + (live[it] ? t : 0);
-    m[it] = -INFINITY;
-    l[it] = 0.f;
+    // a sink is a score without a key: it starts the running maximum and counts once in the sum
+    m[it] = sink != nullptr ? sink[head[it]] : -INFINITY;
+    l[it] = sink != nullptr ? 1.f : 0.f;
 #pragma unroll
     for (int r = 0; r < RPL; ++r) acc[it][r] = 0.f;
   }
@@ -446,7 +455,7 @@ extern "C" int yk_latent_tile_tokens(int n_heads) {
 
 extern "C" int yk_latent_attention(const float* q_lat, const void* pages, int dtype, const int32_t* tiles, int n_tiles,
                                    const int32_t* block_table, int table_width, int page_size, int n_heads, int kv_rank,
-                                   int rot_dim, float scale, float* out, hipStream_t stream) {
+                                   int rot_dim, float scale, const float* sink, float* out, hipStream_t stream) {
   YK_REQUIRE(n_tiles >= 0 && n_heads > 0 && kv_rank > 0 && rot_dim >= 0 && page_size > 0 && table_width > 0,
              "latent_attention: bad sizes");
   YK_REQUIRE(kv_rank <= 16 * kWave, "latent_attention: latents of more than 1,024 elements are not offered");
@@ -474,7 +483,7 @@ extern "C" int yk_latent_attention(const float* q_lat, const void* pages, int dt
                             static_cast<int>(lds)) != hipSuccess)                                                      \
       return yk_fail("latent_attention: the key block does not fit in LDS");                                           \
     kern<<<grid, 64 * kLatWaves, lds, stream>>>(q_lat, static_cast<const T*>(pages), tiles, block_table, table_width,  \
-                                                page_size, n_heads, hpg, kv_rank, rot_dim, scale, KB, pad, out);       \
+                                                page_size, n_heads, hpg, kv_rank, rot_dim, scale, KB, pad, sink, out);       \
     return yk_check_launch("latent_attention");                                                                        \
   }
 #define YK_RPL(T)                      \
@@ -522,7 +531,8 @@ template <int KS, int CT>
 __global__ __launch_bounds__(256, 1) void latent_attention_mfma_kernel(
     const float* __restrict__ q_lat, const bf16_t* __restrict__ kpages, const bf16_t* __restrict__ vpages,
     const int32_t* __restrict__ tiles, int n_tiles, const int32_t* __restrict__ block_table, int table_width, int page_size,
-    int n_heads, float scale_log2, int n_splits, float* __restrict__ out, float* __restrict__ ws_o, float* __restrict__ ws_ml) {
+    int n_heads, float scale_log2, int n_splits, const float* __restrict__ sink, float* __restrict__ out, float* __restrict__ ws_o,
+    float* __restrict__ ws_ml) {
   constexpr int WIDTH = 32 * KS, RANK = 16 * CT;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x % kWave;
   const int tile_i = blockIdx.x * 4 + wave;
@@ -624,6 +634,8 @@ __global__ __launch_bounds__(256, 1) void latent_attention_mfma_kernel(
   // acc[ct][j]: latent column 16 ct + 4 g + j of this lane's column r
   if (n_splits == 1) {
     if (!col_ok) return;
+    // the sink joins the sum of weights at the end (every column has seen a key: m is finite)
+    if (sink != nullptr) l += __builtin_amdgcn_exp2f(sink[head] * 1.4426950408889634f - m);
     const float inv = 1.f / l;
     float* o = out + (static_cast<size_t>(tok0 + tt) * n_heads + head) * RANK + 4 * g;
 #pragma unroll
@@ -646,7 +658,8 @@ __global__ __launch_bounds__(256, 1) void latent_attention_mfma_kernel(
 // column's parts are asked for together
 __global__ __launch_bounds__(128) void latent_attention_merge_kernel(const float* __restrict__ ws_o, const float* __restrict__ ws_ml,
                                                                      const int32_t* __restrict__ tiles, int n_heads, int rank,
-                                                                     int n_splits, float* __restrict__ out) {
+                                                                     int n_splits, const float* __restrict__ sink,
+                                                                     float* __restrict__ out) {
   __shared__ float w[256];
   __shared__ float inv_den;
   const int tile_i = blockIdx.x, chunk = blockIdx.y, r = blockIdx.z;
@@ -667,6 +680,7 @@ __global__ __launch_bounds__(128) void latent_attention_merge_kernel(const float
       den = fmaf(ws, ws_ml[((part0 + s) * 16 + r) * 2 + 1], den);
     }
     den = wave_sum(den);
+    if (sink != nullptr) den += exp2f(sink[head] * 1.4426950408889634f - m_max);
     if (threadIdx.x == 0) inv_den = 1.f / den;
   }
   __syncthreads();
@@ -690,11 +704,13 @@ __global__ __launch_bounds__(128) void latent_attention_merge_kernel(const float
   }
 }
 
-// sizes the matrix-core form is built for: (page row, latent) = (576, 512), (320, 256), (160, 128), (96, 64)
+// sizes the matrix-core form is built for: (page row, latent) = (576, 512), (320, 256), (160, 128), (96, 64), and
+// rows that are the latent alone (no rotated part) of 512, 256, 128 or 64 elements
 extern "C" int yk_latent_mfma_ok(int kv_rank, int rot_dim, int page_size) {
   const int w = kv_rank + rot_dim;
   const bool size_ok = (w == 576 && kv_rank == 512) || (w == 320 && kv_rank == 256) || (w == 160 && kv_rank == 128) ||
-                       (w == 96 && kv_rank == 64);
+                       (w == 96 && kv_rank == 64) ||
+                       (rot_dim == 0 && (kv_rank == 512 || kv_rank == 256 || kv_rank == 128 || kv_rank == 64));
   return size_ok && page_size % 32 == 0 ? 1 : 0;
 }
 
@@ -709,7 +725,7 @@ extern "C" size_t yk_latent_mfma_workspace(int n_tiles, int n_heads, int kv_rank
 
 extern "C" int yk_latent_attention_mfma(const float* q_lat, const void* kpages, const void* vpages, const int32_t* tiles,
                                         int n_tiles, const int32_t* block_table, int table_width, int page_size, int n_heads,
-                                        int kv_rank, int rot_dim, float scale, int n_splits, float* workspace,
+                                        int kv_rank, int rot_dim, float scale, int n_splits, const float* sink, float* workspace,
                                         size_t workspace_floats, float* out, hipStream_t stream) {
   YK_REQUIRE(yk_latent_mfma_ok(kv_rank, rot_dim, page_size), "latent_attention_mfma: sizes the matrix-core form is not built for");
   YK_REQUIRE(n_tiles >= 0 && n_heads > 0 && table_width > 0 && n_splits >= 1 && n_splits <= 256, "latent_attention_mfma: bad sizes");
@@ -725,16 +741,20 @@ extern "C" int yk_latent_attention_mfma(const float* q_lat, const void* kpages, 
   if (kv_rank + rot_dim == 32 * KS && kv_rank == 16 * CT) {                                                                  \
     latent_attention_mfma_kernel<KS, CT><<<grid, 256, 0, stream>>>(                                                          \
         q_lat, static_cast<const bf16_t*>(kpages), static_cast<const bf16_t*>(vpages), tiles, n_tiles, block_table,          \
-        table_width, page_size, n_heads, scale_log2, n_splits, out, ws_o, ws_ml);                                            \
+        table_width, page_size, n_heads, scale_log2, n_splits, sink, out, ws_o, ws_ml);                                            \
     if (yk_check_launch("latent_attention_mfma") != 0) return -1;                                                            \
   }
   YK_CASE(18, 32)
   YK_CASE(10, 16)
   YK_CASE(5, 8)
   YK_CASE(3, 4)
+  YK_CASE(16, 32)
+  YK_CASE(8, 16)
+  YK_CASE(4, 8)
+  YK_CASE(2, 4)
 #undef YK_CASE
   if (n_splits > 1) {
-    latent_attention_merge_kernel<<<dim3(n_tiles, chunks, 16), 128, 0, stream>>>(ws_o, ws_ml, tiles, n_heads, kv_rank, n_splits, out);
+    latent_attention_merge_kernel<<<dim3(n_tiles, chunks, 16), 128, 0, stream>>>(ws_o, ws_ml, tiles, n_heads, kv_rank, n_splits, sink, out);
     return yk_check_launch("latent_attention_merge");
   }
   return 0;

@@ -31,7 +31,7 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(
   for (int e = threadIdx.x; e < n_experts; e += blockDim.x) cnt[e] = 0;
   __syncthreads();
   for (int i = threadIdx.x; i < n_pairs; i += blockDim.x) {
-    int id = token_ids[i / top];
+    int id = token_ids != nullptr ? token_ids[i / top] : i / top;  // (no ids: the table has a row per token of the step)
     id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
     const int e = table[static_cast<size_t>(id) * top + i % top];
     atomicAdd(&cnt[e], 1);
@@ -66,7 +66,7 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(
   }
   __syncthreads();
   for (int i = threadIdx.x; i < n_pairs; i += blockDim.x) {
-    int id = token_ids[i / top];
+    int id = token_ids != nullptr ? token_ids[i / top] : i / top;  // (no ids: the table has a row per token of the step)
     id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
     const int e = table[static_cast<size_t>(id) * top + i % top];
     const int at = atomicAdd(&cnt[e], 1);
@@ -90,6 +90,115 @@ extern "C" int yk_moe_route(const int32_t* token_ids, const int32_t* table, int 
   moe_route_kernel<<<1, 1024, lds, stream>>>(token_ids, table, vocab, top, n_experts, n_pairs, tile_rows, order,
                                              slot_expert, tiles, n_tiles, yk_moe_max_tiles(n_pairs, n_experts, tile_rows));
   return yk_check_launch("moe_route");
+}
+
+// ------------------------------------------------------------------------ a learned router
+// Per token: the `top` experts with the largest logits (ties: the lower number), their numbers into choice
+// [tokens][top], and the token's row once per chosen expert, multiplied by that expert's score sigmoid(logit), into xs
+// [tokens * top][hidden]: the score weighs what the expert reads, not what it returns.  A workgroup a token; its
+// first wave chooses.
+template <typename T>
+__global__ __launch_bounds__(256) void moe_router_topk_kernel(const float* __restrict__ logits, int logits_stride, int n_experts, int top,
+                                                              const T* __restrict__ x, int x_stride, int hidden,
+                                                              int32_t* __restrict__ choice, T* __restrict__ xs) {
+  extern __shared__ float sel[];  // [top] scores, then [top] numbers (as ints)
+  int* sel_e = reinterpret_cast<int*>(sel + top);
+  const int n = blockIdx.x, lane = threadIdx.x;
+  const float* row = logits + static_cast<size_t>(n) * logits_stride;
+  if (threadIdx.x < kWave) {
+    for (int k = 0; k < top; ++k) {
+      float best = -INFINITY;
+      int best_e = 0x7fffffff;
+      for (int e = lane; e < n_experts; e += kWave) {
+        bool taken = false;
+        for (int j = 0; j < k; ++j) taken |= sel_e[j] == e;
+        const float v = row[e];
+        // (a NaN is never larger: such a row falls back on the lowest free numbers)
+        if (!taken && (v > best || (best_e == 0x7fffffff) || (v == best && e < best_e))) {
+          best = v;
+          best_e = e;
+        }
+      }
+      // the wave's best: the largest value, among equals the lowest number
+      for (int off = kWave / 2; off > 0; off /= 2) {
+        const float ov = __shfl_xor(best, off, kWave);
+        const int oe = __shfl_xor(best_e, off, kWave);
+        if (oe != 0x7fffffff && (best_e == 0x7fffffff || ov > best || (ov == best && oe < best_e))) {
+          best = ov;
+          best_e = oe;
+        }
+      }
+      if (lane == 0) {
+        sel_e[k] = best_e;
+        sel[k] = 1.f / (1.f + expf(-best));
+        choice[static_cast<size_t>(n) * top + k] = best_e;
+      }
+      __builtin_amdgcn_wave_barrier();
+      __threadfence_block();
+    }
+  }
+  __syncthreads();
+  const T* src = x + static_cast<size_t>(n) * x_stride;
+  for (int c = threadIdx.x; c < hidden; c += blockDim.x) {
+    const float v = to_f32<T>(src[c]);
+    for (int k = 0; k < top; ++k) xs[(static_cast<size_t>(n) * top + k) * hidden + c] = from_f32<T>(v * sel[k]);
+  }
+}
+
+extern "C" int yk_moe_router_topk(const float* logits, int logits_stride, int n_experts, int top, const void* x, int x_stride, int dtype,
+                                  int hidden, int32_t* choice, void* xs, int n_tokens, hipStream_t stream) {
+  YK_REQUIRE(n_tokens >= 0 && n_experts >= 1 && top >= 1 && top <= n_experts && top <= 64 && hidden > 0 && x_stride >= hidden &&
+                 logits_stride >= n_experts,
+             "moe_router_topk: bad sizes (up to 64 experts a token)");
+  if (n_tokens == 0) return 0;
+  const size_t lds = 2 * static_cast<size_t>(top) * sizeof(float);
+  if (dtype == YK_F32)
+    moe_router_topk_kernel<float><<<n_tokens, 256, lds, stream>>>(logits, logits_stride, n_experts, top, static_cast<const float*>(x), x_stride,
+                                                                  hidden, choice, static_cast<float*>(xs));
+  else if (dtype == YK_BF16)
+    moe_router_topk_kernel<bf16_t><<<n_tokens, 256, lds, stream>>>(logits, logits_stride, n_experts, top, static_cast<const bf16_t*>(x), x_stride,
+                                                                   hidden, choice, static_cast<bf16_t*>(xs));
+  else
+    return yk_fail("moe_router_topk: unsupported dtype");
+  return yk_check_launch("moe_router_topk");
+}
+
+// out[n, :] = dense[n, :] (a tensor, a product's unreduced slices, or nothing) + weight * the sum of the token's `top`
+// rows of rows [tokens * top][width]: what a mixture adds to the stream, as one float32 tensor
+template <typename TD>
+__global__ void moe_combine_kernel(const TD* __restrict__ dense, int n_splits, size_t split_stride, int round_sum,
+                                   const float* __restrict__ rows, int top, float weight, float* __restrict__ out, int width,
+                                   size_t total) {
+  for (size_t i = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; i < total;
+       i += static_cast<size_t>(gridDim.x) * blockDim.x) {
+    const size_t n = i / width;
+    const int c = static_cast<int>(i % width);
+    float d = 0.f;
+    if (dense != nullptr) {
+      for (int s = 0; s < n_splits; ++s) d += to_f32<TD>(dense[s * split_stride + i]);
+      d = as_output(d, round_sum);
+    }
+    float e = 0.f;
+    for (int k = 0; k < top; ++k) e += rows[(n * top + k) * width + c];
+    out[i] = fmaf(weight, e, d);
+  }
+}
+
+extern "C" int yk_moe_combine(const void* dense, int dense_dtype, int n_splits, int round_sum, const float* rows, int top,
+                              float weight, float* out, int n_tokens, int width, hipStream_t stream) {
+  YK_REQUIRE(n_tokens >= 0 && width > 0 && top >= 1 && n_splits >= 1 && (n_splits == 1 || dense_dtype == YK_F32), "moe_combine: bad sizes");
+  if (n_tokens == 0) return 0;
+  const size_t total = static_cast<size_t>(n_tokens) * width;
+  const int grid = static_cast<int>(std::min<size_t>((total + 255) / 256, 1 << 20));
+  if (dense == nullptr || dense_dtype == YK_F32)
+    moe_combine_kernel<float><<<grid, 256, 0, stream>>>(static_cast<const float*>(dense), n_splits, total, round_sum, rows, top,
+                                                        weight, out, width, total);
+  else if (dense_dtype == YK_BF16)
+    moe_combine_kernel<bf16_t><<<grid, 256, 0, stream>>>(static_cast<const bf16_t*>(dense), n_splits, total, round_sum, rows, top,
+                                                         weight, out, width, total);
+  else
+    return yk_fail("moe_combine: unsupported dtype");
+  return yk_check_launch("moe_combine");
 }
 
 // ---------------------------------------------------------------- float32 FMA products

@@ -3,7 +3,9 @@
 //   S <- diag(a_t) S                       a_t: one decay for the head, or one per key channel (row of S)
 //   u  = v_t                               plain write
 //   u  = beta_t (v_t - S^T k_t)            delta rule
-//   S <- S + k_t u^T,   o_t = S^T q_t      (the read-out sees the token's own write)
+//   u  = dt_t v_t                          a write as strong as the token's step (state-space duality: with the head's
+//                                          decay exp(-exp(A_log) dt_t), dt_t = softplus(x + dt_bias), q = C, k = B)
+//   S <- S + k_t u^T,   o_t = S^T q_t      (the read-out sees the token's own write; + skip_h v_t where a skip is given)
 //
 // The columns of S never meet: column e needs k_t, q_t, a_t, beta_t and its own v_t[e] only.  So a
 // column lives in the registers of a group of TPC lanes (lane s of the group holds the rows s,
@@ -95,7 +97,8 @@ __global__ __launch_bounds__(256) void linear_state_scan_kernel(
     const int32_t* __restrict__ seq_qstart, const int32_t* __restrict__ seq_qlen, const int32_t* __restrict__ state_slots,
     float q_scale, float unit_eps, int decay_mode, const float* __restrict__ decay, int decay_stride, int decay_col,
     const float* __restrict__ decay_p0, const float* __restrict__ decay_p1, float tau, const float* __restrict__ beta,
-    int beta_stride, int beta_col, int chunk, float* __restrict__ out) {
+    int beta_stride, int beta_col, int chunk, float* __restrict__ out, int q_col, int k_col, int v_col, int write_mode,
+    const float* __restrict__ skip) {
   extern __shared__ float lds[];
   constexpr int DP = TPC * kScanRows;  // padded key channels
   constexpr int DS = DP + 4;           // a staged row's stride: rows of different tokens then start in different banks
@@ -114,7 +117,8 @@ __global__ __launch_bounds__(256) void linear_state_scan_kernel(
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave, n_waves = blockDim.x / kWave;
   const int q0 = seq_qstart[seq], ql = seq_qlen[seq];
   float* S_head = state + (static_cast<size_t>(state_slots[seq]) * n_heads + h) * dim * vdim;
-  const bool delta = beta != nullptr;
+  const bool delta = write_mode == 1;
+  const float skip_h = skip != nullptr ? skip[h] : 0.f;
 
   float S[kScanRows];
 #pragma unroll
@@ -122,7 +126,6 @@ __global__ __launch_bounds__(256) void linear_state_scan_kernel(
     const int i = sub * kScanRows + r;
     S[r] = has_col && i < dim ? S_head[static_cast<size_t>(i) * vdim + col] : 0.f;
   }
-  const int kd = n_kv * dim;
   for (int t0 = 0; t0 < ql; t0 += chunk) {
     const int nt = min(chunk, ql - t0);
     __syncthreads();  // the chunk before has been read
@@ -140,7 +143,7 @@ __global__ __launch_bounds__(256) void linear_state_scan_kernel(
         const int v = threadIdx.x + j * 256;
         const int item = v / P8, c = 8 * (v % P8), t = item >> 1, is_k = item & 1;
         if (v < n_qk && c < dim)
-          scan_load8<T>(qkv + static_cast<size_t>(q0 + t0 + t) * qkv_stride + (is_k ? kd : 0) + kvh * dim + c, qk[j]);
+          scan_load8<T>(qkv + static_cast<size_t>(q0 + t0 + t) * qkv_stride + (is_k ? k_col : q_col) + kvh * dim + c, qk[j]);
         else {
 #pragma unroll
           for (int e = 0; e < 8; ++e) qk[j][e] = 0.f;
@@ -166,7 +169,7 @@ __global__ __launch_bounds__(256) void linear_state_scan_kernel(
         for (int j = 0; j < 8; ++j) {
           const int i = i0 + threadIdx.x + j * 256;
           const int t = i / cols_per_block, c = col0 + i % cols_per_block;
-          vv[j] = i < n_v && c < vdim ? to_f32<T>(qkv[static_cast<size_t>(q0 + t0 + t) * qkv_stride + 2 * kd + h * vdim + c]) : 0.f;
+          vv[j] = i < n_v && c < vdim ? to_f32<T>(qkv[static_cast<size_t>(q0 + t0 + t) * qkv_stride + v_col + h * vdim + c]) : 0.f;
         }
         if (i0 + 8 * 256 < n_v) {
 #pragma unroll
@@ -216,8 +219,9 @@ __global__ __launch_bounds__(256) void linear_state_scan_kernel(
         }
       }
       if (threadIdx.x < nt) {
-        if (decay_mode == 0) as[threadIdx.x] = expf(-expf(decay_p0[h]) * scan_softplus(s_dec + decay_p1[h]));
-        bs[threadIdx.x] = delta ? 1.f / (1.f + expf(-s_beta)) : 1.f;
+        const float step = decay_mode == 0 ? scan_softplus(s_dec + decay_p1[h]) : 1.f;
+        if (decay_mode == 0) as[threadIdx.x] = expf(-expf(decay_p0[h]) * step);
+        bs[threadIdx.x] = delta ? 1.f / (1.f + expf(-s_beta)) : (write_mode == 2 ? step : 1.f);
       }
     } else {
     // q and k of the chunk's tokens to LDS, every load of a thread asked for before the first is used
@@ -232,7 +236,7 @@ __global__ __launch_bounds__(256) void linear_state_scan_kernel(
           const int i = i0 + j * blockDim.x;
           const int item = i / DP, c = i % DP, t = item >> 1, is_k = item & 1;
           x[j] = i < total && c < dim
-                     ? to_f32<T>(qkv[static_cast<size_t>(q0 + t0 + t) * qkv_stride + (is_k ? kd : 0) + kvh * dim + c])
+                     ? to_f32<T>(qkv[static_cast<size_t>(q0 + t0 + t) * qkv_stride + (is_k ? k_col : q_col) + kvh * dim + c])
                      : 0.f;
         }
 #pragma unroll
@@ -267,13 +271,13 @@ __global__ __launch_bounds__(256) void linear_state_scan_kernel(
     }
     for (int i = threadIdx.x; i < nt * cols_per_block; i += blockDim.x) {
       const int t = i / cols_per_block, c = col0 + i % cols_per_block;
-      vs[i] = c < vdim ? to_f32<T>(qkv[static_cast<size_t>(q0 + t0 + t) * qkv_stride + 2 * kd + h * vdim + c]) : 0.f;
+      vs[i] = c < vdim ? to_f32<T>(qkv[static_cast<size_t>(q0 + t0 + t) * qkv_stride + v_col + h * vdim + c]) : 0.f;
     }
     for (int t = threadIdx.x; t < nt; t += blockDim.x) {
       const size_t n = static_cast<size_t>(q0 + t0 + t);
-      if (decay_mode == 0)
-        as[t] = expf(-expf(decay_p0[h]) * scan_softplus(decay[n * decay_stride + decay_col + h] + decay_p1[h]));
-      bs[t] = delta ? 1.f / (1.f + expf(-beta[n * beta_stride + beta_col + h])) : 1.f;
+      const float step = decay_mode == 0 ? scan_softplus(decay[n * decay_stride + decay_col + h] + decay_p1[h]) : 1.f;
+      if (decay_mode == 0) as[t] = expf(-expf(decay_p0[h]) * step);
+      bs[t] = delta ? 1.f / (1.f + expf(-beta[n * beta_stride + beta_col + h])) : (write_mode == 2 ? step : 1.f);
     }
     }
     __syncthreads();
@@ -355,7 +359,8 @@ __global__ __launch_bounds__(256) void linear_state_scan_kernel(
       const float sq = column_sum<TPC>((pq[0] + pq[1]) + (pq[2] + pq[3]));
       float u = v_t;
       if (delta) u = b_t * (u - column_sum<TPC>((pk[0] + pk[1]) + (pk[2] + pk[3])));
-      const float so = fmaf(u, kq_t, sq);
+      else u *= b_t;  // (1 for plain writes)
+      const float so = fmaf(skip_h, v_t, fmaf(u, kq_t, sq));
 #pragma unroll
       for (int r = 0; r < kScanRows; ++r) S[r] = fmaf(kr[r], u, S[r]);
       if (has_col && sub == 0) out[(static_cast<size_t>(q0 + t0 + t) * n_heads + h) * vdim + col] = so;
@@ -370,16 +375,22 @@ __global__ __launch_bounds__(256) void linear_state_scan_kernel(
 
 // decay_mode 0: one decay per head from decay[n, decay_col + h], p0 = A_log [heads], p1 = dt_bias [heads];
 // decay_mode 1: one per key channel from decay[n, decay_col + h * dim + i], p0 = bias [heads * dim], tau.
-// beta null: plain writes; else the delta rule with beta = sigmoid(beta[n, beta_col + h]).  unit_eps < 0: q
-// and k are taken as they are.
+// write_mode 0: plain writes; 1: the delta rule with beta = sigmoid(beta[n, beta_col + h]); 2: u = dt v with the
+// step dt = softplus(decay[n, decay_col + h] + p1[h]) that the head's decay is made of (decay_mode 0 only).
+// unit_eps < 0: q and k are taken as they are.  q_col, k_col, v_col: where the kv_heads' queries and keys and the
+// heads' values start in a row of qkv.  skip [heads] or null: o += skip[h] v.
 extern "C" int yk_linear_state_scan(const void* qkv, int qkv_stride, int dtype, int n_heads, int n_kv, int dim, int vdim,
                                     float* state, const int32_t* seq_qstart, const int32_t* seq_qlen,
                                     const int32_t* state_slots, int n_seqs, int n_tokens, float q_scale, float unit_eps, int decay_mode,
                                     const float* decay, int decay_stride, int decay_col, const float* decay_p0,
                                     const float* decay_p1, float tau, const float* beta, int beta_stride, int beta_col,
-                                    float* out, hipStream_t stream) {
+                                    float* out, int q_col, int k_col, int v_col, int write_mode, const float* skip,
+                                    hipStream_t stream) {
   YK_REQUIRE(n_seqs >= 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0 && dim > 0 && vdim > 0, "linear_state_scan: bad sizes");
-  YK_REQUIRE(qkv_stride >= 2 * n_kv * dim + n_heads * vdim, "linear_state_scan: rows shorter than q, k and v");
+  YK_REQUIRE(q_col >= 0 && k_col >= 0 && v_col >= 0 && qkv_stride >= std::max(std::max(q_col, k_col) + n_kv * dim, v_col + n_heads * vdim),
+             "linear_state_scan: rows shorter than q, k and v");
+  YK_REQUIRE(write_mode == 0 || (write_mode == 1 && beta != nullptr) || (write_mode == 2 && decay_mode == 0),
+             "linear_state_scan: the delta rule needs beta, a write by the step the decay per head");
   YK_REQUIRE(decay_mode == 0 || decay_mode == 1, "linear_state_scan: unknown kind of decay");
   YK_REQUIRE(decay != nullptr && decay_p0 != nullptr && (decay_mode == 1 || decay_p1 != nullptr), "linear_state_scan: the decay's inputs are missing");
   YK_REQUIRE(decay_mode == 0 || tau > 0.f, "linear_state_scan: tau must be positive");
@@ -403,7 +414,7 @@ extern "C" int yk_linear_state_scan(const void* qkv, int qkv_stride, int dtype, 
   const size_t lds = chunk * per_token;
   YK_REQUIRE(lds <= 128 * 1024, "linear_state_scan: the staged tokens do not fit in LDS");
   auto al16 = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
-  const bool vec = dim % 8 == 0 && qkv_stride % 8 == 0 && (n_kv * dim) % 8 == 0 && al16(qkv) && chunk * dp <= 8192 &&
+  const bool vec = dim % 8 == 0 && qkv_stride % 8 == 0 && q_col % 8 == 0 && k_col % 8 == 0 && al16(qkv) && chunk * dp <= 8192 &&
                    (decay_mode == 0 || (decay_stride % 4 == 0 && decay_col % 4 == 0 && al16(decay) && al16(decay_p0)));
 #define YK_LAUNCH(T, TPC)                                                                                                       \
   {                                                                                                                             \
@@ -414,7 +425,8 @@ extern "C" int yk_linear_state_scan(const void* qkv, int qkv_stride, int dtype, 
       return yk_fail("linear_state_scan: the staged tokens do not fit in LDS");                                                 \
     kern<<<grid, threads, lds, stream>>>(static_cast<const T*>(qkv), qkv_stride, n_heads, n_kv, dim, vdim, state, seq_qstart,   \
                                          seq_qlen, state_slots, q_scale, unit_eps, decay_mode, decay, decay_stride, decay_col,  \
-                                         decay_p0, decay_p1, tau, beta, beta_stride, beta_col, chunk, out);                     \
+                                         decay_p0, decay_p1, tau, beta, beta_stride, beta_col, chunk, out, q_col, k_col,       \
+                                         v_col, write_mode, skip);                                                              \
     return yk_check_launch("linear_state_scan");                                                                                \
   }
 #define YK_TPC(T)                   \
@@ -435,38 +447,54 @@ extern "C" int yk_linear_state_scan(const void* qkv, int qkv_stride, int dtype, 
 }
 
 // --------------------------------------------------------------- the read-out's norm and gate
-// a wave per (token, head): y = o / sqrt(mean(o^2) + eps) * w * silu(gate)
+// a wave per (token, part of vdim elements): y = o / sqrt(mean(o^2) + eps) * w * silu(gate), or, gate_first, the gate
+// before the norm: y = g / sqrt(mean(g^2) + eps) * w with g = o * silu(gate).  w_stride 0: one weight of vdim elements
+// for every part; vdim: a weight of n_heads * vdim elements.
 template <typename TW, typename TG, typename TO>
 __global__ __launch_bounds__(256) void gated_head_norm_kernel(const float* __restrict__ o, const TW* __restrict__ w, float eps,
                                                               const TG* __restrict__ gate, int gate_stride, int gate_col,
-                                                              int n_heads, int vdim, TO* __restrict__ out, size_t total) {
+                                                              int n_heads, int vdim, TO* __restrict__ out, size_t total,
+                                                              int w_stride, int gate_first) {
   const size_t item = blockIdx.x * static_cast<size_t>(blockDim.x / kWave) + threadIdx.x / kWave;
   if (item >= total) return;
   const int lane = threadIdx.x % kWave;
   const size_t n = item / n_heads;
   const int h = static_cast<int>(item % n_heads);
   const float* row = o + item * vdim;
+  const TG* g = gate + n * gate_stride + gate_col + h * vdim;
+  const TW* wp = w + static_cast<size_t>(h) * w_stride;
   float ss = 0.f;
+  if (gate_first) {
+    for (int c = lane; c < vdim; c += kWave) {
+      const float v = row[c] * act_silu(to_f32<TG>(g[c]));
+      ss = fmaf(v, v, ss);
+    }
+    const float inv = 1.f / sqrtf(wave_sum(ss) / static_cast<float>(vdim) + eps);
+    for (int c = lane; c < vdim; c += kWave)
+      out[item * vdim + c] = from_f32<TO>(row[c] * act_silu(to_f32<TG>(g[c])) * inv * to_f32<TW>(wp[c]));
+    return;
+  }
   for (int c = lane; c < vdim; c += kWave) ss = fmaf(row[c], row[c], ss);
   const float inv = 1.f / sqrtf(wave_sum(ss) / static_cast<float>(vdim) + eps);
-  const TG* g = gate + n * gate_stride + gate_col + h * vdim;
   for (int c = lane; c < vdim; c += kWave)
-    out[item * vdim + c] = from_f32<TO>(row[c] * inv * to_f32<TW>(w[c]) * act_silu(to_f32<TG>(g[c])));
+    out[item * vdim + c] = from_f32<TO>(row[c] * inv * to_f32<TW>(wp[c]) * act_silu(to_f32<TG>(g[c])));
 }
 
 extern "C" int yk_gated_head_norm(const float* o, const void* w, int w_dtype, float eps, const void* gate, int gate_dtype,
                                   int gate_stride, int gate_col, int n_heads, int vdim, void* out, int out_dtype, int n_tokens,
-                                  hipStream_t stream) {
+                                  int w_per_part, int gate_first, hipStream_t stream) {
   YK_REQUIRE(n_tokens >= 0 && n_heads > 0 && vdim > 0 && gate_stride >= gate_col + n_heads * vdim, "gated_head_norm: bad sizes");
   YK_REQUIRE(gate_dtype == out_dtype, "gated_head_norm: the gate comes in the output's dtype");
   if (n_tokens == 0) return 0;
   const size_t total = static_cast<size_t>(n_tokens) * n_heads;
   const int grid = static_cast<int>((total + 3) / 4);
+  const int w_stride = w_per_part ? vdim : 0;
 #define YK_CASE(WD, TW, OD, TO)                                                                                       \
   if (w_dtype == WD && out_dtype == OD) {                                                                             \
     gated_head_norm_kernel<TW, TO, TO><<<grid, 256, 0, stream>>>(o, static_cast<const TW*>(w), eps,                   \
                                                                  static_cast<const TO*>(gate), gate_stride, gate_col, \
-                                                                 n_heads, vdim, static_cast<TO*>(out), total);        \
+                                                                 n_heads, vdim, static_cast<TO*>(out), total, w_stride, \
+                                                                 gate_first);                                         \
     return yk_check_launch("gated_head_norm");                                                                        \
   }
   YK_CASE(YK_F32, float, YK_F32, float)

@@ -168,7 +168,9 @@ class DecoderModel:
         """Run the step's tokens; returns float32 logits [wanted rows, vocab]."""
         first = self.blocks[self.spec.run_order[0].layer]
         begin = getattr(self.embedding, "begin", None)
-        if begin is not None:
+        if getattr(self.embedding, "needs_positions", False):
+            residual, delta = self.embedding.forward(ctx.arrays["token_ids"], ctx.arrays["positions"]), None
+        elif begin is not None:
             residual, delta = begin(ctx.arrays["token_ids"], bool(getattr(first, "takes_embedded_rows", False)))
         else:
             residual, delta = self.embedding.forward(ctx.arrays["token_ids"]), None

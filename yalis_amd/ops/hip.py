@@ -48,7 +48,7 @@ def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
 _SIGNATURES = {
     "yk_abi_version": ([], _c_int),
     "yk_cache_tiled": ([_c_int, _c_int, _c_int], _c_int),
-    "yk_embed": ([_vp, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _vp], _c_int),
+    "yk_embed": ([_vp, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _vp, _vp, _c_int, _vp], _c_int),
     "yk_add_rmsnorm": (
         [_vp, _vp, _c_int, _c_int, _c_int, _vp, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _vp, _c_int, _vp],
         _c_int,
@@ -73,11 +73,13 @@ _SIGNATURES = {
     ),
     "yk_attn_masked": (
         [_vp, _c_int, _vp, _vp, _vp, _c_int, _vp, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float,
-         _c_float, _c_int, _c_int, _c_int, _vp, _vp, _c_int, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _vp],
+         _c_float, _c_int, _c_int, _c_int, _vp, _vp, _c_int, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _vp,
+         _c_int, _vp],
         _c_int,
     ),
     "yk_attn_finish": (
-        [_vp, _c_int, _vp, _c_int, _c_int, _c_int, _vp, _vp, _c_int, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _vp],
+        [_vp, _c_int, _vp, _c_int, _c_int, _c_int, _vp, _vp, _c_int, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
+         _vp],
         _c_int,
     ),
     "yk_causal_conv": ([_vp, _c_int, _c_int, _vp, _vp, _c_int, _vp, _vp, _vp, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _vp], _c_int),
@@ -97,28 +99,31 @@ _SIGNATURES = {
     "yk_latent_mfma_tile_tokens": ([_c_int], _c_int),
     "yk_latent_mfma_workspace": ([_c_int, _c_int, _c_int, _c_int], _c_size_t),
     "yk_latent_attention_mfma": (
-        [_vp, _vp, _vp, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _vp, _c_size_t, _vp, _vp],
+        [_vp, _vp, _vp, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _vp, _vp, _c_size_t, _vp, _vp],
         _c_int,
     ),
     "yk_head_linear": (
         [_vp, _c_int, _c_int, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _vp, _vp, _c_int, _vp, _c_int, _c_int,
-         _c_int, _c_int, _vp],
+         _c_int, _c_int, _c_int, _vp],
         _c_int,
     ),
     "yk_head_linear_mfma_ok": ([_c_int, _c_int, _c_int], _c_int),
     "yk_head_linear_mfma": (
         [_vp, _c_int, _c_int, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _vp, _vp, _c_int, _vp, _c_int, _c_int,
-         _c_int, _c_int, _vp],
+         _c_int, _c_int, _c_int, _vp],
         _c_int,
     ),
     "yk_latent_tile_tokens": ([_c_int], _c_int),
-    "yk_latent_attention": ([_vp, _vp, _c_int, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _vp, _vp], _c_int),
+    "yk_latent_attention": ([_vp, _vp, _c_int, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _vp, _vp, _vp], _c_int),
     "yk_linear_state_scan": (
         [_vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _vp, _vp, _vp, _c_int, _c_int, _c_float, _c_float, _c_int, _vp, _c_int,
-         _c_int, _vp, _vp, _c_float, _vp, _c_int, _c_int, _vp, _vp],
+         _c_int, _vp, _vp, _c_float, _vp, _c_int, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _vp, _vp],
         _c_int,
     ),
-    "yk_gated_head_norm": ([_vp, _vp, _c_int, _c_float, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _c_int, _c_int, _vp], _c_int),
+    "yk_gated_head_norm": (
+        [_vp, _vp, _c_int, _c_float, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _vp],
+        _c_int,
+    ),
     "yk_conv_state_push": ([_vp, _c_int, _c_int, _vp, _vp, _vp, _vp, _c_int, _c_int, _c_int, _vp], _c_int),
     "yk_rglru_gates": ([_vp, _c_int, _vp, _vp, _vp, _vp, _vp, _c_int, _c_float, _vp, _vp, _c_int, _c_int, _c_int, _vp, _vp, _vp], _c_int),
     "yk_rglru_gates_mfma_ok": ([_c_int, _c_int], _c_int),
@@ -129,6 +134,8 @@ _SIGNATURES = {
     "yk_rglru_scan": ([_vp, _vp, _vp, _c_int, _vp, _c_int, _c_int, _vp, _vp, _vp, _vp, _vp, _vp, _c_int, _c_int, _c_int, _vp], _c_int),
     "yk_moe_max_tiles": ([_c_int, _c_int, _c_int], _c_int),
     "yk_moe_mfma_ok": ([_c_int, _c_int, _c_int], _c_int),
+    "yk_moe_router_topk": ([_vp, _c_int, _c_int, _c_int, _vp, _c_int, _c_int, _c_int, _vp, _vp, _c_int, _vp], _c_int),
+    "yk_moe_combine": ([_vp, _c_int, _c_int, _c_int, _vp, _c_int, _c_float, _vp, _c_int, _c_int, _vp], _c_int),
     "yk_moe_route": ([_vp, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _vp, _vp, _vp, _vp], _c_int),
     "yk_moe_gate_up": (
         [_vp, _c_int, _c_int, _vp, _c_int, _vp, _vp, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float,
@@ -202,7 +209,7 @@ _LATER_SIGNATURES = {
         "yk_probe_mfma_bf16": ([_c_int, _c_int, _vp, _vp], _c_int),
     },
 }
-_ABI = 18
+_ABI = 19
 
 # Rows of x up to which the hand-written matrix-core kernel runs a bfloat16 product;
 # above it the vendor library does.
@@ -476,14 +483,22 @@ class HipOps:
         return 2 if workgroups >= 1024 or fewest_keys >= 1024 else 1
 
     # ------------------------------------------------------------------ embedding
-    def embed(self, token_ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
+    def embed(self, token_ids: torch.Tensor, table: torch.Tensor, positions=None, position_table=None) -> torch.Tensor:
+        """float32 rows table[id] (+ position_table[position], a learned vector per absolute position, summed in
+        float32)."""
         self._rows(table, "embed table")
         n = token_ids.numel()
+        if position_table is not None:
+            self._rows(position_table, "position table")
+            if (position_table.dtype != table.dtype or position_table.shape[1] != table.shape[1] or not position_table.is_contiguous()
+                    or positions is None or positions.numel() != n or positions.dtype != torch.int32):
+                raise KernelError("embed: the position table has the embedding table's dtype and width, and every token an int32 position")
         out = torch.empty((n, table.shape[1]), dtype=torch.float32, device=table.device)
         self._check(
             self.lib.yk_embed(
                 token_ids.data_ptr(), table.data_ptr(), _code(table.dtype), out.data_ptr(), n,
-                table.shape[1], table.shape[0], self._stream(),
+                table.shape[1], table.shape[0], _ptr(positions) if position_table is not None else None, _ptr(position_table),
+                0 if position_table is None else position_table.shape[0], self._stream(),
             )
         )
         return out
@@ -1201,13 +1216,18 @@ class HipOps:
 
     def attention_masked(self, q, n_heads, n_kv, head_dim, value_dim, k_cache, v_cache, page_size, scale, ctx, group,
                          window: int = 0, keep_first: int = 0, softcap: float = 0.0, value_rotation=None,
-                         gate=None, gate_col: int = 0) -> torch.Tensor:
+                         gate=None, gate_col: int = 0, gate_elems: int = 1, distance_bias=None) -> torch.Tensor:
         """softmax over the keys j <= p with (p - j < window or j < keep_first) of q . k * scale
         (squashed by ``softcap`` * tanh(s / ``softcap``) when set), times the values [N, n_heads *
         value_dim]; then, with ``value_rotation``, every head's output turned back by its token's
         position, and, with ``gate`` (the projection, a tensor or ``SplitSum``, whose columns
-        ``gate_col`` + h hold the heads' gates), multiplied by the sigmoid of its gate."""
+        ``gate_col`` + h hold the heads' gates), multiplied by the sigmoid of its gate (``gate_elems`` = value_dim:
+        a gate per output element, in the columns ``gate_col`` + h * value_dim + d).  ``distance_bias`` (float32
+        [distances, n_heads]): row min(p - j, distances - 1) is added to the scaled scores of head h."""
         self._rows(q, "queries")
+        if distance_bias is not None and (distance_bias.dtype != torch.float32 or distance_bias.dim() != 2 or not distance_bias.is_contiguous()
+                                          or distance_bias.shape[1] != n_heads or distance_bias.shape[0] < 1):
+            raise KernelError("attention_masked: the distance bias is contiguous float32 [distances, heads]")
         n = q.shape[0]
         bt = ctx.arrays[f"block_table_g{group}"]
         if tuple(k_cache.shape[1:]) != (n_kv, page_size, head_dim) or tuple(v_cache.shape[1:]) != (n_kv, value_dim, page_size):
@@ -1225,12 +1245,14 @@ class HipOps:
                 int(keep_first or 0), int(self.masked_pages_tiled(q.dtype, head_dim, value_dim, page_size)),
                 None if vr is None else vr.cos.data_ptr(), None if vr is None else vr.sin.data_ptr(),
                 int(bool(vr is not None and vr.interleaved)), 0 if vr is None else vr.cos.shape[0],
-                _ptr(gsrc), 0 if gsrc is None else _code(gsrc.dtype), gsplits, ground, gstride, int(gate_col), self._stream(),
+                _ptr(gsrc), 0 if gsrc is None else _code(gsrc.dtype), gsplits, ground, gstride, int(gate_col), int(gate_elems),
+                _ptr(distance_bias), 0 if distance_bias is None else distance_bias.shape[0], self._stream(),
             )
         )
         return out
 
-    def attention_finish(self, out, positions, n_heads, value_dim, value_rotation=None, gate=None, gate_col: int = 0):
+    def attention_finish(self, out, positions, n_heads, value_dim, value_rotation=None, gate=None, gate_col: int = 0,
+                         gate_elems: int = 1):
         """In place on an attention's output [N, n_heads * value_dim]: the turn back by the position
         and the gate, as ``attention_masked`` applies them itself."""
         n = out.shape[0]
@@ -1241,7 +1263,8 @@ class HipOps:
                 out.data_ptr(), _code(out.dtype), positions.data_ptr(), n, value_dim, n_heads,
                 None if vr is None else vr.cos.data_ptr(), None if vr is None else vr.sin.data_ptr(),
                 int(bool(vr is not None and vr.interleaved)), 0 if vr is None else vr.cos.shape[0],
-                _ptr(gsrc), 0 if gsrc is None else _code(gsrc.dtype), gsplits, ground, gstride, int(gate_col), self._stream(),
+                _ptr(gsrc), 0 if gsrc is None else _code(gsrc.dtype), gsplits, ground, gstride, int(gate_col), int(gate_elems),
+                self._stream(),
             )
         )
         return out
@@ -1392,11 +1415,12 @@ class HipOps:
         return w.transpose(1, 2).contiguous()
 
     def head_linear(self, x, w, n_heads, in_dim, out_dim, out_dtype, tail=0, rotation=None, positions=None, gate=None, gate_col=0,
-                    w_t=None):
+                    w_t=None, gate_elems=1):
         """Per head, out[n, h, :out_dim] = x[n, h, :in_dim] . w[h] with w [heads, in_dim, out_dim]
         (float32 sums).  ``tail`` further elements of every head of x follow the product in the output,
         turned by the token's position (``rotation``, ``positions``); ``gate`` [N, >= gate_col + heads]:
-        head h's output is multiplied by sigmoid(gate[n, gate_col + h]).  ``w_t`` (``head_weights_transposed``):
+        head h's output is multiplied by sigmoid(gate[n, gate_col + h]) (``gate_elems`` = out_dim: element o of it by
+        sigmoid(gate[n, gate_col + h * out_dim + o])).  ``w_t`` (``head_weights_transposed``):
         with it, products of many tokens run on the matrix cores (a float32 input as two bfloat16 parts)."""
         self._rows(x, "head_linear input")
         n = x.shape[0]
@@ -1405,8 +1429,8 @@ class HipOps:
         out = torch.empty((n, n_heads * (out_dim + tail)), dtype=out_dtype, device=x.device)
         if gate is not None:
             self._rows(gate, "head_linear gate")
-            if gate.shape[0] != n or gate.shape[1] < gate_col + n_heads:
-                raise KernelError("head_linear: the gate's rows do not hold a column per head")
+            if gate_elems not in (1, out_dim) or gate.shape[0] != n or gate.shape[1] < gate_col + n_heads * gate_elems:
+                raise KernelError("head_linear: the gate's rows do not hold a column per head (or per output element)")
         cos = sin = None
         inter = 0
         if tail:
@@ -1422,12 +1446,12 @@ class HipOps:
             self._check(self.lib.yk_head_linear_mfma(
                 x.data_ptr(), x.stride(0), _code(x.dtype), w_t.data_ptr(), out.data_ptr(), _code(out_dtype), n_heads, in_dim, out_dim,
                 tail, _ptr(positions), _ptr(cos), _ptr(sin), inter, _ptr(gate), 0 if gate is None else _code(gate.dtype),
-                0 if gate is None else gate.stride(0), gate_col, n, self._stream()))
+                0 if gate is None else gate.stride(0), gate_col, int(gate_elems), n, self._stream()))
             return out
         self._check(self.lib.yk_head_linear(
             x.data_ptr(), x.stride(0), _code(x.dtype), w.data_ptr(), _code(w.dtype), out.data_ptr(), _code(out_dtype), n_heads, in_dim,
             out_dim, tail, _ptr(positions), _ptr(cos), _ptr(sin), inter, _ptr(gate), 0 if gate is None else _code(gate.dtype),
-            0 if gate is None else gate.stride(0), gate_col, n, self._stream()))
+            0 if gate is None else gate.stride(0), gate_col, int(gate_elems), n, self._stream()))
         return out
 
     def latent_attention_on_matrix_cores(self, act_dtype: torch.dtype, kv_rank: int, rot_dim: int, page_size: int) -> bool:
@@ -1447,13 +1471,16 @@ class HipOps:
         return max(1, min(-(-512 // max(waves, 1)), max(1, -(-max_ctx // 32) // 4), 64))
 
     def latent_attention(self, q_lat, pages, n_heads, kv_rank, rot_dim, scale, ctx, group, page_size, tiles=None, values=None,
-                         splits: Optional[int] = None) -> torch.Tensor:
+                         splits: Optional[int] = None, sink=None) -> torch.Tensor:
         """Causal softmax attention of ``q_lat`` (float32 [N, heads * (kv_rank + rot_dim)]) over the page
         rows [c | kr] of each token's request: scores q . row * scale, the result sum_j p_j c_j as
         float32 [N, heads * kv_rank].  ``tiles``: the step's spans cut into ``latent_tile_tokens`` tokens
-        (rows of request, first token, count, first position)."""
+        (rows of request, first token, count, first position).  ``sink`` (float32 [heads]): exp(sink_h) joins the
+        softmax's denominator of head h, a score with no key and no value."""
         n = q_lat.shape[0]
         width = kv_rank + rot_dim
+        if sink is not None and (sink.dtype != torch.float32 or sink.numel() != n_heads or not sink.is_contiguous()):
+            raise KernelError("latent_attention: the sinks are contiguous float32, one per head")
         if q_lat.dtype != torch.float32 or not q_lat.is_contiguous() or q_lat.shape[1] != n_heads * width:
             raise KernelError("latent_attention: queries are contiguous float32 [N, heads * (kv_rank + rot_dim)]")
         if pages.dim() != 4 or pages.shape[1] != 1 or pages.shape[2] != page_size or pages.shape[3] != width or not pages.is_contiguous():
@@ -1473,12 +1500,12 @@ class HipOps:
             ws = self._ws(floats) if floats else None
             self._check(self.lib.yk_latent_attention_mfma(
                 q_lat.data_ptr(), pages.data_ptr(), values.data_ptr(), tiles.data_ptr(), tiles.shape[0], bt.data_ptr(), bt.shape[1],
-                page_size, n_heads, kv_rank, rot_dim, float(scale), splits, _ptr(ws), 0 if ws is None else ws.numel(), out.data_ptr(),
+                page_size, n_heads, kv_rank, rot_dim, float(scale), splits, _ptr(sink), _ptr(ws), 0 if ws is None else ws.numel(), out.data_ptr(),
                 self._stream()))
             return out
         self._check(self.lib.yk_latent_attention(
             q_lat.data_ptr(), pages.data_ptr(), _code(pages.dtype), tiles.data_ptr(), tiles.shape[0], bt.data_ptr(), bt.shape[1],
-            page_size, n_heads, kv_rank, rot_dim, float(scale), out.data_ptr(), self._stream()))
+            page_size, n_heads, kv_rank, rot_dim, float(scale), _ptr(sink), out.data_ptr(), self._stream()))
         return out
 
     # ---------------------------------------------------------------- a matrix per head as the memory
@@ -1493,20 +1520,32 @@ class HipOps:
             x.data_ptr(), x.stride(0), _code(x.dtype), state.data_ptr(), a["seq_qstart"].data_ptr(), a["seq_qlen"].data_ptr(),
             a["state_slots"].data_ptr(), a["seq_qstart"].numel(), state.shape[1], channels, self._stream()))
 
-    def linear_state_scan(self, qkv, n_heads, n_kv, dim, vdim, state, ctx, q_scale=1.0, unit_eps=None, decay=None, beta=None):
+    def linear_state_scan(self, qkv, n_heads, n_kv, dim, vdim, state, ctx, q_scale=1.0, unit_eps=None, decay=None, beta=None,
+                          columns=None, skip=None):
         """The recurrence S <- diag(a) S; u = v or beta (v - S^T k); S += k u^T; o = S^T q over each
         request's span, S [slots, heads, dim, vdim] float32 updated in place.  ``qkv`` [N, >= 2 * kv_heads *
         dim + heads * vdim]: columns [q | k | v].  ``unit_eps``: q and k are divided by sqrt(sum of squares +
         unit_eps) first; q is multiplied by ``q_scale``.  ``decay``: ("head", x, col, A_log, dt_bias): a =
         exp(-exp(A_log) softplus(x[:, col + h] + dt_bias)); ("channel", z, col, bias, tau): a_i = sigmoid(z[:,
         col + h * dim + i] + bias)^(1 / tau); x, z float32.  ``beta``: (x, col) -> sigmoid(x[:, col + h]), or
-        None for plain writes.  Returns o float32 [N, heads * vdim]."""
+        None for plain writes, or "step": u = dt v with the step dt = softplus(x[:, col + h] + dt_bias) of the head's
+        decay.  ``columns`` = (q, k, v): where the kv heads' queries and keys and the heads' values start in a row
+        (default 0, n_kv * dim, 2 * n_kv * dim).  ``skip`` (float32 [heads]): o += skip_h v.  Returns o float32 [N,
+        heads * vdim]."""
         self._rows(qkv, "linear_state_scan input")
         n = qkv.shape[0]
         if state.dtype != torch.float32 or not state.is_contiguous() or tuple(state.shape[1:]) != (n_heads, dim, vdim):
             raise KernelError(f"linear_state_scan: state {tuple(state.shape)} does not hold {n_heads} matrices of {dim} x {vdim}")
         kind, src, col = decay[0], decay[1], int(decay[2])
         need = n_heads if kind == "head" else n_heads * dim
+        write_mode = 0 if beta is None else (2 if isinstance(beta, str) else 1)
+        if isinstance(beta, str) and (beta != "step" or kind != "head"):
+            raise KernelError("linear_state_scan: a write by the step goes with the decay per head")
+        if write_mode != 1:
+            beta = None
+        q_col, k_col, v_col = columns if columns is not None else (0, n_kv * dim, 2 * n_kv * dim)
+        if skip is not None and (skip.dtype != torch.float32 or skip.numel() != n_heads or not skip.is_contiguous()):
+            raise KernelError("linear_state_scan: the skip is contiguous float32, one number per head")
         for t, what, cols in ((src, "decay", col + need),) + (((beta[0], "beta", int(beta[1]) + n_heads),) if beta is not None else ()):
             if t.dtype != torch.float32 or t.dim() != 2 or t.stride(1) != 1 or t.shape[0] != n or t.shape[1] < cols:
                 raise KernelError(f"linear_state_scan: the {what}'s input must be float32 rows of at least {cols} columns")
@@ -1527,22 +1566,27 @@ class HipOps:
             a["seq_qlen"].data_ptr(), a["state_slots"].data_ptr(), a["seq_qstart"].numel(), n, float(q_scale),
             -1.0 if unit_eps is None else float(unit_eps), 0 if kind == "head" else 1, src.data_ptr(), src.stride(0), col,
             p0.data_ptr(), _ptr(p1), tau, None if beta is None else beta[0].data_ptr(), 0 if beta is None else beta[0].stride(0),
-            0 if beta is None else int(beta[1]), out.data_ptr(), self._stream()))
+            0 if beta is None else int(beta[1]), out.data_ptr(), int(q_col), int(k_col), int(v_col), write_mode, _ptr(skip),
+            self._stream()))
         return out
 
-    def gated_head_norm(self, o, weight, eps, gate, gate_col, n_heads, vdim, out_dtype) -> torch.Tensor:
+    def gated_head_norm(self, o, weight, eps, gate, gate_col, n_heads, vdim, out_dtype, gate_first: bool = False) -> torch.Tensor:
         """Per head, o / sqrt(mean(o^2) + eps) * weight * silu(gate[:, gate_col + h * vdim + .]); ``o`` float32
-        [N, heads * vdim], ``weight`` [vdim] shared by the heads."""
+        [N, heads * vdim], ``weight`` [vdim] shared by the heads, or [heads * vdim].  The "heads" are whatever equal
+        parts of a row are normed each by its own root mean square.  ``gate_first``: the gate comes before the
+        norm, rms(o * silu(gate)) * weight."""
         n = o.shape[0]
         self._rows(gate, "gated_head_norm gate")
-        if o.dtype != torch.float32 or not o.is_contiguous() or o.shape[1] != n_heads * vdim or weight.numel() != vdim or not weight.is_contiguous():
-            raise KernelError("gated_head_norm: o is contiguous float32 [N, heads * vdim], the weight [vdim]")
+        if o.dtype != torch.float32 or not o.is_contiguous() or o.shape[1] != n_heads * vdim or weight.numel() not in (vdim, n_heads * vdim) \
+                or not weight.is_contiguous():
+            raise KernelError("gated_head_norm: o is contiguous float32 [N, heads * vdim], the weight [vdim] or [heads * vdim]")
         if gate.dtype != out_dtype or gate.shape[0] != n or gate.shape[1] < gate_col + n_heads * vdim:
             raise KernelError("gated_head_norm: the gate does not fit")
         out = torch.empty((n, n_heads * vdim), dtype=out_dtype, device=o.device)
         self._check(self.lib.yk_gated_head_norm(
             o.data_ptr(), weight.data_ptr(), _code(weight.dtype), float(eps), gate.data_ptr(), _code(gate.dtype), gate.stride(0),
-            gate_col, n_heads, vdim, out.data_ptr(), _code(out_dtype), n, self._stream()))
+            gate_col, n_heads, vdim, out.data_ptr(), _code(out_dtype), n, int(weight.numel() != vdim or n_heads == 1),
+            int(bool(gate_first)), self._stream()))
         return out
 
     # spans of more than this many tokens are scanned in chunks (cut by the caller)
@@ -1605,14 +1649,21 @@ class HipOps:
     def moe_experts(self, x, token_ids, table, w_gate_up, w_down, activation) -> torch.Tensor:
         """Every token through the experts its id names in ``table`` [vocab, top]: returns float32
         rows [N * top, hidden], row n * top + k the output of token n's k-th expert (uncombined).
-        ``w_gate_up`` [experts, 2, ff, hidden] (gate rows, then up rows), ``w_down`` [experts, hidden, ff]."""
+        ``w_gate_up`` [experts, 2, ff, hidden] (gate rows, then up rows), ``w_down`` [experts, hidden, ff].
+        ``token_ids`` None: ``table`` has a row per token of the step (a router's choice) and ``x`` a row per
+        (token, k) already, [N * top, hidden] (what ``moe_router_topk`` returns)."""
         self._rows(x, "expert input")
-        n, hidden = x.shape
         vocab, top = table.shape
+        if token_ids is None:
+            n, hidden, x_top = vocab, x.shape[1], 1  # x_top: how many pairs share a row of x
+            if x.shape[0] != n * top:
+                raise KernelError("moe: with a choice per token the input has a row per (token, choice)")
+        else:
+            (n, hidden), x_top = x.shape, top
         experts, two, ff, hid = w_gate_up.shape
         if two != 2 or hid != hidden or tuple(w_down.shape) != (experts, hidden, ff) or not w_gate_up.is_contiguous() or not w_down.is_contiguous():
             raise KernelError("moe: expert weights must be contiguous [experts, 2, ff, hidden] and [experts, hidden, ff]")
-        if table.dtype != torch.int32 or not table.is_contiguous() or token_ids.dtype != torch.int32 or token_ids.numel() != n:
+        if table.dtype != torch.int32 or not table.is_contiguous() or (token_ids is not None and (token_ids.dtype != torch.int32 or token_ids.numel() != n)):
             raise KernelError("moe: the table and the token ids are int32, one id per row")
         kind, p0, p1 = self.gated_kind(activation)
         pairs = n * top
@@ -1627,7 +1678,7 @@ class HipOps:
         order, slot_expert = ints[:pairs], ints[pairs: 2 * pairs]
         tiles, n_tiles = ints[2 * pairs: 2 * pairs + 3 * max_tiles], ints[2 * pairs + 3 * max_tiles:]
         self._check(
-            self.lib.yk_moe_route(token_ids.data_ptr(), table.data_ptr(), vocab, top, experts, n, tile_rows, order.data_ptr(),
+            self.lib.yk_moe_route(_ptr(token_ids), table.data_ptr(), vocab, top, experts, n, tile_rows, order.data_ptr(),
                                   slot_expert.data_ptr(), tiles.data_ptr(), n_tiles.data_ptr(), self._stream())
         )
         bf = torch.bfloat16
@@ -1638,7 +1689,7 @@ class HipOps:
             gu = torch.empty((pairs, 2 * ff), dtype=bf, device=dev)
             self._check(
                 self.lib.yk_gemm_tile_grouped(
-                    x.data_ptr(), x.stride(0), order.data_ptr(), top, w_gate_up.data_ptr(), 2 * ff * hidden, hidden, gu.data_ptr(),
+                    x.data_ptr(), x.stride(0), order.data_ptr(), x_top, w_gate_up.data_ptr(), 2 * ff * hidden, hidden, gu.data_ptr(),
                     _BF16, 2 * ff, None, tiles.data_ptr(), n_tiles.data_ptr(), max_tiles, 2 * ff, hidden, self._stream(),
                 )
             )
@@ -1654,7 +1705,7 @@ class HipOps:
         self._check(
             self.lib.yk_moe_gate_up(
                 x.data_ptr(), x.stride(0), _code(x.dtype), w_gate_up.data_ptr(), _code(w_gate_up.dtype), order.data_ptr(),
-                slot_expert.data_ptr(), tiles.data_ptr(), n_tiles.data_ptr(), tile_rows, max_tiles, pairs, top, hidden, ff,
+                slot_expert.data_ptr(), tiles.data_ptr(), n_tiles.data_ptr(), tile_rows, max_tiles, pairs, x_top, hidden, ff,
                 kind, p0, p1, y.data_ptr(), self._stream(),
             )
         )
@@ -1665,6 +1716,40 @@ class HipOps:
             )
         )
         return rows
+
+    def moe_router_topk(self, logits, x, top: int, experts: Optional[int] = None):
+        """From a router's float32 ``logits`` [N, >= experts] (``experts``: how many of a row's columns are experts; the
+        rest is padding): the ``top`` experts with the largest logits of every token
+        (int32 [N, top]; among equals the lower number) and the token's row of ``x`` once per chosen expert times the
+        expert's score sigmoid(logit) ([N * top, hidden] in x's dtype): the score weighs the expert's input."""
+        self._rows(x, "router input")
+        self._rows(logits, "router logits")
+        n = logits.shape[0]
+        experts = logits.shape[1] if experts is None else int(experts)
+        if logits.dtype != torch.float32 or experts > logits.shape[1] or x.shape[0] != n or not 1 <= top <= min(experts, 64):
+            raise KernelError("moe_router_topk: logits are float32 [N, >= experts], top between 1 and min(experts, 64)")
+        choice = torch.empty((n, top), dtype=torch.int32, device=x.device)
+        xs = torch.empty((n * top, x.shape[1]), dtype=x.dtype, device=x.device)
+        self._check(self.lib.yk_moe_router_topk(logits.data_ptr(), logits.stride(0), experts, int(top), x.data_ptr(), x.stride(0), _code(x.dtype),
+                                                x.shape[1], choice.data_ptr(), xs.data_ptr(), n, self._stream()))
+        return choice, xs
+
+    def moe_combine(self, dense, rows, top: int, weight: float = 1.0) -> torch.Tensor:
+        """float32 [N, width]: ``dense`` (a tensor, a ``SplitSum`` or None) + weight * the sum of each token's ``top``
+        consecutive rows of ``rows`` (float32 [N * top, width])."""
+        if rows.dtype != torch.float32 or not rows.is_contiguous() or rows.dim() != 2 or rows.shape[0] % top:
+            raise KernelError("moe_combine: the experts' rows are contiguous float32 [N * top, width]")
+        n, width = rows.shape[0] // top, rows.shape[1]
+        n_splits, round_sum, src = 1, 0, dense
+        if isinstance(dense, SplitSum):
+            dense.check_live()
+            n_splits, round_sum, src = dense.n_splits, dense.round_sum, dense.tensor
+        if dense is not None and (tuple(dense.shape) != (n, width) or not src.is_contiguous()):
+            raise KernelError(f"moe_combine: the dense part {tuple(dense.shape)} does not match the rows {(n, width)}")
+        out = torch.empty((n, width), dtype=torch.float32, device=rows.device)
+        self._check(self.lib.yk_moe_combine(_ptr(src), 0 if src is None else _code(src.dtype), n_splits, round_sum, rows.data_ptr(),
+                                            int(top), float(weight), out.data_ptr(), n, width, self._stream()))
+        return out
 
     # ------------------------------------------------------------------- sampling
     def argmax(self, logits: torch.Tensor) -> torch.Tensor:

@@ -24,10 +24,17 @@ their position and a head's output is turned back by the query's position, so th
 the output depends on distances), softcap (scores squashed to softcap * tanh(s / softcap)),
 keep_first (that many first keys stay visible below the window), gate (a tensor name below the
 prefix, [num_heads, hidden]: a head's output is multiplied by the sigmoid of its row's product with
-the mixer's input).
+the mixer's input; with gate_per "element" the tensor is [num_heads * value_dim, hidden] and the
+concatenated heads are multiplied element by element), distance_bias ({"name": tensor below the
+prefix, [buckets, num_heads]; "far": D; "buckets": B or None, the tensor's rows}: a learned number per
+head added to the scaled score of a key n positions back, row bucket(n) of the tensor with bucket(n) =
+n below B/2 and min(B - 1, B/2 + floor(ln(n / (B/2)) / ln(D / (B/2)) * (B - B/2))) from there on, so
+that distances up to B/2 have a row each and the rows beyond cover distances that grow
+geometrically up to D).  A layer may have no position encoding at all (``position`` None).
 """
 from __future__ import annotations
 
+import math
 from typing import Dict, Mapping
 
 import numpy as np
@@ -79,9 +86,15 @@ class Attention(Mixer):
         self.softcap = float(params.get("softcap") or 0.0)
         self.keep_first = int(params.get("keep_first") or 0)
         self.gate_name = params.get("gate")
+        self.gate_per = params.get("gate_per", "head")
+        if self.gate_per not in ("head", "element"):
+            raise ValueError(f"{self.prefix}: gate_per is 'head' or 'element', got {self.gate_per!r}")
+        self.gate_elems = self.value_dim if self.gate_per == "element" else 1
+        self.distance_bias = params.get("distance_bias")
+        self.bias_by_distance = None
         self.masked = bool(
             self.value_dim != self.head_dim or self.qk_norm or self.value_norm_eps is not None or self.value_rotation is not None
-            or self.softcap or self.keep_first or self.gate_name
+            or self.softcap or self.keep_first or self.gate_name or self.distance_bias
         )
         self.w_qn = self.w_kn = None
         if self.masked:
@@ -94,7 +107,9 @@ class Attention(Mixer):
             # the matrix-core kernels take these options too, where they take the sizes (bfloat16, keys and
             # values of 64 or 128 elements alike); everything else runs on the general float32-arithmetic kernel
             can = getattr(rt.ops, "attention_can_rotate", None)
-            self.on_matrix_cores = bool(can is not None and self.value_dim == self.head_dim and can(rt.act_dtype, self.head_dim) is True)
+            # (a bias per distance is the general kernel's alone)
+            self.on_matrix_cores = bool(can is not None and self.value_dim == self.head_dim and can(rt.act_dtype, self.head_dim) is True
+                                        and not self.distance_bias)
             if self.on_matrix_cores:
                 self._tile_sizes(rt)
             return
@@ -135,7 +150,11 @@ class Attention(Mixer):
             if self.projects_kv:
                 specs[f"{self.prefix}.{self.qk_norm['k']}"] = TensorSpec((self.head_dim,), "float", ("one_plus_normal", 0.1))
         if self.gate_name:
-            specs[f"{self.prefix}.{self.gate_name}"] = TensorSpec((self.n_heads, self.hidden))
+            specs[f"{self.prefix}.{self.gate_name}"] = TensorSpec((self.n_heads * self.gate_elems, self.hidden))
+        if self.distance_bias:
+            rows = self.distance_bias.get("buckets")
+            specs[f"{self.prefix}.{self.distance_bias['name']}"] = TensorSpec((int(rows or 16), self.n_heads), "float", ("normal", 1.0),
+                                                                              free_axes=() if rows else (0,))
         if self.bias:
             for which, spec in list(specs.items()):
                 specs[self._bias_name(which)] = TensorSpec((spec.shape[0],), "float", ("normal", 0.02))
@@ -164,6 +183,8 @@ class Attention(Mixer):
             if self.qk_norm:
                 self.w_qn = tensors[f"{self.prefix}.{self.qk_norm['q']}"]
                 self.w_kn = tensors[f"{self.prefix}.{self.qk_norm['k']}"] if self.projects_kv else self.w_qn
+            if self.distance_bias:
+                self.bias_by_distance = self._bias_by_distance(tensors[f"{self.prefix}.{self.distance_bias['name']}"])
             return
         if self.projects_kv:
             self.w_qkv = torch.cat([q, tensors[self.names["k"]], tensors[self.names["v"]]], dim=0).contiguous()
@@ -180,6 +201,28 @@ class Attention(Mixer):
                 self.b_q = b("q")
             self.b_o = b("o")
 
+    @staticmethod
+    def distance_bucket(n: int, buckets: int, far: float) -> int:
+        half = buckets // 2
+        if n < half:
+            return n
+        return min(buckets - 1, half + int(math.floor(math.log(n / half) / math.log(far / half) * (buckets - half))))
+
+    def _bias_by_distance(self, table: torch.Tensor) -> torch.Tensor:
+        """The table [buckets, heads] spread out as float32 [distances, heads], a row per distance a key can have:
+        up to the window, or to where the last bucket begins (every larger distance reads the last row)."""
+        buckets, far = int(table.shape[0]), float(self.distance_bias["far"])
+        if buckets < 2 or far <= buckets // 2:
+            raise ValueError(f"{self.prefix}: a distance bias needs at least two buckets and far={far} beyond the {buckets // 2} exact ones")
+        reach = self.rt.max_positions if not self.window else min(int(self.window), self.rt.max_positions)
+        rows = []
+        for n in range(max(reach, 1)):
+            rows.append(self.distance_bucket(n, buckets, far))
+            if rows[-1] == buckets - 1:
+                break
+        index = torch.tensor(rows, dtype=torch.long, device=table.device)
+        return table.float().index_select(0, index).contiguous()
+
     def kv_need(self) -> KVNeed:
         return KVNeed(self.n_kv, self.head_dim, self.window, None if self.value_dim == self.head_dim else self.value_dim,
                       self.keep_first if self.window else 0)
@@ -187,7 +230,7 @@ class Attention(Mixer):
     def products(self):
         hd, kd = self.n_heads * self.head_dim, self.n_kv * self.head_dim
         if self.masked:
-            rows = hd + (kd + self.n_kv * self.value_dim if self.projects_kv else 0) + (self.n_heads if self.gate_name else 0)
+            rows = hd + (kd + self.n_kv * self.value_dim if self.projects_kv else 0) + (self.n_heads * self.gate_elems if self.gate_name else 0)
             return ((rows + (-rows % 16), self.hidden), (self.hidden, self.n_heads * self.value_dim))
         return ((hd + 2 * kd if self.projects_kv else hd, self.hidden), (self.hidden, hd))
 
@@ -254,12 +297,13 @@ class Attention(Mixer):
             )
             if self.value_rotation is not None or self.gate_name:
                 ops.attention_finish(out, ctx.arrays["positions"], self.n_heads, self.value_dim, self.value_rotation,
-                                     gate=proj if self.gate_name else None, gate_col=gate_col)
+                                     gate=proj if self.gate_name else None, gate_col=gate_col, gate_elems=self.gate_elems)
             return ops.linear(out, self.w_o, self.rt.act_dtype, partial_ok=True)
         out = ops.attention_masked(
             q, self.n_heads, self.n_kv, self.head_dim, self.value_dim, k_cache, v_cache, self.rt.page_size, self.scale, ctx,
             site.group, window=0 if self.window is None else int(self.window), keep_first=self.keep_first,
             softcap=self.softcap, value_rotation=self.value_rotation, gate=proj if self.gate_name else None, gate_col=gate_col,
+            gate_elems=self.gate_elems, distance_bias=self.bias_by_distance,
         )
         return ops.linear(out, self.w_o, self.rt.act_dtype, partial_ok=True)
 

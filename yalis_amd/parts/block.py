@@ -2,7 +2,8 @@
 
 "prenorm" is the reference's sequential pre-norm block
 (yalis/external/model.py:414-439 with parallel_residual=False and identity
-post-norms): x = x + mixer(norm_1(x)); x = x + feed_forward(norm_2(x)).
+post-norms): x = x + mixer(norm_1(x)); x = x + feed_forward(norm_2(x)); a layer may leave the
+feed-forward and its norm out.
 
 The residual stream is float32.  A block receives the residual and the previous
 block's not-yet-added contribution ``delta``; each norm kernel adds the pending
@@ -19,11 +20,13 @@ class PreNormBlock(Block):
     roles = {
         "mixer_norm": ("norm", True),
         "mixer": ("mixer", True),
-        "feed_forward_norm": ("norm", True),
-        "feed_forward": ("feed_forward", True),
+        "feed_forward_norm": ("norm", False),
+        "feed_forward": ("feed_forward", False),
     }
 
-    def __init__(self, mixer_norm, mixer, feed_forward_norm, feed_forward):
+    def __init__(self, mixer_norm, mixer, feed_forward_norm=None, feed_forward=None):
+        if (feed_forward is None) != (feed_forward_norm is None):
+            raise ValueError("a prenorm block has a feed-forward and its norm, or neither")
         self.mixer_norm = mixer_norm
         self.mixer = mixer
         self.feed_forward_norm = feed_forward_norm
@@ -36,6 +39,8 @@ class PreNormBlock(Block):
     def forward(self, residual, delta, ctx, site):
         h = self.mixer_norm.add_norm(residual, delta)
         a = self.mixer.forward(h, ctx, site)
+        if self.feed_forward is None:  # a layer that is its mixer alone: the mixer's output waits for the next norm
+            return a
         h = self.feed_forward_norm.add_norm(residual, a)
         return self.feed_forward.forward(h, ctx)
 

@@ -50,6 +50,37 @@ class TokenEmbedding(Part):
         return self.forward(token_ids), None
 
 
+@register_embedding("token_position_embedding")
+class TokenPositionEmbedding(TokenEmbedding):
+    """The token's row plus a learned vector for its absolute position (not scaled), summed in float32.
+
+    params: name, position_name (a table [max_positions, hidden]), vocab_size, hidden_size, max_positions."""
+
+    graph_capturable = True
+    needs_positions = True
+
+    def __init__(self, params, rt: Runtime):
+        super().__init__(params, rt)
+        self.position_name = params["position_name"]
+        self.max_positions = int(params["max_positions"])
+        self.position_table = None
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        return {self.name: TensorSpec((self.vocab, self.hidden)), self.position_name: TensorSpec((self.max_positions, self.hidden))}
+
+    def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
+        self.table = tensors[self.name]
+        self.position_table = tensors[self.position_name].contiguous()
+
+    def forward(self, token_ids: torch.Tensor, positions: torch.Tensor = None) -> torch.Tensor:
+        if positions is None:
+            raise ValueError("this embedding adds a vector per position: it needs the tokens' positions")
+        return self.rt.ops.embed(token_ids, self.table, positions=positions, position_table=self.position_table)
+
+    def begin(self, token_ids: torch.Tensor, lazily: bool, positions: torch.Tensor = None):
+        return self.forward(token_ids, positions), None
+
+
 @register_head("lm_head")
 class LMHead(Part):
     """params: name, tied_to (name of the embedding table, or None), vocab_size,

@@ -19,7 +19,12 @@ W_uv is applied to the kv_rank-wide result of each head.
 
 params: prefix, hidden_size, num_heads, head_dim, rot_dim, value_dim, kv_rank, q_rank, scale,
 latent_eps (of the two latent norms), gate (tensor name below the prefix or None), position (a
-PartSpec whose ``rotation()`` covers exactly rot_dim elements), names (optional overrides).
+PartSpec whose ``rotation()`` covers exactly rot_dim elements; None with rot_dim 0: no rotated part,
+the page row is the latent alone and positions enter through the causal mask only), gate_per
+("head": the gate's tensor has a row per head; "element": one per head and value element, and the
+concatenated heads are multiplied element by element), sink (tensor name below the prefix or None:
+a learned number per head whose exponential joins the softmax's denominator, a score that has no
+key and no value and is not scaled), names (optional overrides).
 """
 from __future__ import annotations
 
@@ -59,21 +64,27 @@ class LatentAttention(Mixer):
         self.eps = float(params["latent_eps"])
         self.gate_name = params.get("gate")
         self.projects_kv = bool(params.get("projects_kv", True))
-        pos: PartSpec = params["position"]
-        self.position = POSITIONS.get(pos.kind)(pos.params, rt)
-        self.rotation = self.position.rotation()
-        if self.rotation is None or self.rotation.rotary_dim != self.rot_dim:
+        self.sink_name = params.get("sink")
+        self.gate_per = params.get("gate_per", "head")
+        if self.gate_per not in ("head", "element"):
+            raise ValueError(f"{self.prefix}: gate_per is 'head' or 'element', got {self.gate_per!r}")
+        self.gate_elems = self.value_dim if self.gate_per == "element" else 1
+        pos: PartSpec = params.get("position")
+        self.position = None if pos is None else POSITIONS.get(pos.kind)(pos.params, rt)
+        self.rotation = None if self.position is None else self.position.rotation()
+        if (self.rot_dim or self.position is not None) and (self.rotation is None or self.rotation.rotary_dim != self.rot_dim):
             raise ValueError(f"{self.prefix}: the position encoding must rotate exactly the rot_dim={self.rot_dim} elements of the rotated part")
         names = {"dq": "dq", "dq_norm": "dq.norm", "uq": "uq", "dkv": "dkv", "dkv_norm": "dkv.norm", "uk": "uk", "uv": "uv", "o": "o"}
         names.update(params.get("names", {}))
         self.names = {k: f"{self.prefix}.{v}" for k, v in names.items()}
         self.w_down = self.w_qn = self.w_kvn = self.w_uq = self.w_uk = self.w_uv_t = self.w_o = self.w_uk_t = self.w_uv = None
+        self.sink = None
         # columns of the stacked down-projection: [dq | dkv (where the layer keeps a cache) | gates], each
         # section starting at a multiple of 8
         up8 = lambda n: n + (-n % 8)
         self.kv_col = up8(self.q_rank)
         self.gate_col = self.kv_col + (up8(self.kv_rank + self.rot_dim) if self.projects_kv else 0)
-        self.down_rows = self.gate_col + (self.n_heads if self.gate_name else 0)
+        self.down_rows = self.gate_col + (self.n_heads * self.gate_elems if self.gate_name else 0)
         self.down_rows += -self.down_rows % 16
         # where the kernel library has its matrix-core attention for these sizes the latent is kept a second
         # time, transposed, in value pages (that form's second product reads a column's slots side by side)
@@ -93,7 +104,9 @@ class LatentAttention(Mixer):
             specs[n["dkv"]] = TensorSpec((self.kv_rank + self.rot_dim, self.hidden))
             specs[n["dkv_norm"]] = TensorSpec((self.kv_rank,), "float", ("one_plus_normal", 0.1))
         if self.gate_name:
-            specs[f"{self.prefix}.{self.gate_name}"] = TensorSpec((H, self.hidden))
+            specs[f"{self.prefix}.{self.gate_name}"] = TensorSpec((H * self.gate_elems, self.hidden))
+        if self.sink_name:
+            specs[f"{self.prefix}.{self.sink_name}"] = TensorSpec((H,), "float", ("normal", 1.0))
         return specs
 
     def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
@@ -109,6 +122,8 @@ class LatentAttention(Mixer):
         parts.append(zeros(self.down_rows - sum(p.shape[0] for p in parts)))
         self.w_down = torch.cat([p for p in parts if p.shape[0]], dim=0).contiguous()
         self.w_qn = tensors[n["dq_norm"]].contiguous()
+        if self.sink_name:
+            self.sink = tensors[f"{self.prefix}.{self.sink_name}"].float().contiguous()
         self.w_uq = tensors[n["uq"]]
         # per head [in][out]: W_uk as it is stored ([head][dim][kv_rank]: out = kv_rank), W_uv transposed
         # ([head][kv_rank][value_dim])
@@ -149,7 +164,8 @@ class LatentAttention(Mixer):
         q_lat = ops.head_linear(q, self.w_uk, self.n_heads, self.head_dim, self.kv_rank, torch.float32, tail=self.rot_dim,
                                 rotation=self.rotation, positions=ctx.arrays["positions"], w_t=self.w_uk_t)
         o_lat = ops.latent_attention(q_lat, pages, self.n_heads, self.kv_rank, self.rot_dim, self.scale, ctx, site.group,
-                                     self.rt.page_size, tiles=ctx.arrays[f"latent_tiles_{self.tile_tokens}"], values=values)
+                                     self.rt.page_size, tiles=ctx.arrays[f"latent_tiles_{self.tile_tokens}"], values=values,
+                                     sink=self.sink)
         o = ops.head_linear(o_lat, self.w_uv_t, self.n_heads, self.kv_rank, self.value_dim, act,
-                            gate=proj if self.gate_name else None, gate_col=self.gate_col, w_t=self.w_uv)
+                            gate=proj if self.gate_name else None, gate_col=self.gate_col, w_t=self.w_uv, gate_elems=self.gate_elems)
         return ops.linear(o, self.w_o, act, partial_ok=True)

@@ -19,6 +19,14 @@ exp(-exp(A_log) softplus(W_a h + dt_bias)).  The convolution's last inputs are a
 
 "gated_linear_attention" (Yang et al., "Gated Linear Attention Transformers with Hardware-Efficient Training"): q times head_dim^-1/2, decay per key
 channel sigmoid(z)^(1/tau) with z = W_a2 (W_a1 h) + b.
+
+"state_space_duality" (Dao and Gu, "Transformers are SSMs: Generalized Models and Efficient Algorithms Through Structured State Space
+Duality"): the same memory read as a selective state space.  One projection gives [z | x | B | C | dt]; x, B and C
+pass a causal convolution per channel with a bias and silu; the step dt = softplus(dt + dt_bias) makes the head's
+decay exp(-exp(A_log) dt) and the strength of its write, S <- a S + dt B x^T (k = B, u = dt x), the read-out is
+S^T C + D x (q = C, a skip per head); B and C are shared by groups of heads.  The read-out is gated first, by
+silu(z), and then normed in ``norm_groups`` equal parts, each by its own root mean square, with a weight as wide as
+the read-out.
 """
 from __future__ import annotations
 
@@ -185,3 +193,88 @@ class GatedLinearAttention(_MatrixStateMixer):
             unit_eps=None, decay=("channel", z, 0, self.b_a2, self.tau), beta=None,
         )
         return self._finish(o, proj, self.gate_col)
+
+
+@register_mixer("state_space_duality")
+class StateSpaceDuality(Mixer):
+    """params: prefix, hidden_size, num_heads, value_dim (a head's channels), state_dim (rows of S), groups (of heads
+    that share B and C), conv_taps, norm_groups, out_norm_eps, names (optional overrides: in, conv, conv_bias, dt_bias,
+    A_log, D, norm, o)."""
+
+    graph_capturable = True
+
+    def __init__(self, params, rt: Runtime):
+        super().__init__(params, rt)
+        self.prefix = params["prefix"]
+        self.hidden = int(params["hidden_size"])
+        self.n_heads = int(params["num_heads"])
+        self.value_dim = int(params["value_dim"])
+        self.state_dim = int(params["state_dim"])
+        self.groups = int(params["groups"])
+        self.taps = int(params["conv_taps"])
+        self.norm_groups = int(params["norm_groups"])
+        self.out_eps = float(params["out_norm_eps"])
+        self.inner = self.n_heads * self.value_dim
+        if self.n_heads % self.groups:
+            raise ValueError(f"{self.prefix}: num_heads={self.n_heads} is not a multiple of groups={self.groups}")
+        if self.inner % self.norm_groups:
+            raise ValueError(f"{self.prefix}: {self.inner} channels do not divide into norm_groups={self.norm_groups} equal parts")
+        self.bc_cols = self.groups * self.state_dim
+        self.conv_cols = self.inner + 2 * self.bc_cols  # [x | B | C]
+        self.main_rows = 2 * self.inner + 2 * self.bc_cols  # [z | x | B | C]; dt follows in the checkpoint's matrix
+        self.w_main = self.w_dt = self.w_conv = self.b_conv = self.dt_bias = self.a_log = self.skip = self.w_norm = self.w_o = None
+
+    def _name(self, short: str) -> str:
+        default = {"conv_bias": "conv.b"}.get(short, short)
+        return f"{self.prefix}.{self.params.get('names', {}).get(short, default)}"
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        H = self.n_heads
+        return {
+            self._name("in"): TensorSpec((self.main_rows + H, self.hidden)),
+            self._name("conv"): TensorSpec((self.conv_cols, self.taps), "float", ("normal", 0.4)),
+            self._name("conv_bias"): TensorSpec((self.conv_cols,), "float", ("normal", 0.1)),
+            self._name("dt_bias"): TensorSpec((H,), "float", ("normal", 0.5)), self._name("A_log"): TensorSpec((H,), "float", ("normal", 0.5)),
+            self._name("D"): TensorSpec((H,), "float", ("one_plus_normal", 0.1)),
+            self._name("norm"): TensorSpec((self.inner,), "float", ("one_plus_normal", 0.1)),
+            self._name("o"): TensorSpec((self.hidden, self.inner)),
+        }
+
+    def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
+        t = lambda short: tensors[self._name(short)]
+        w_in = t("in")
+        self.w_main = _pad_rows([w_in[: self.main_rows]], 16)
+        self.w_dt = _pad_rows([w_in[self.main_rows:]], 16)
+        self.w_conv, self.b_conv = t("conv").contiguous(), t("conv_bias").contiguous()
+        if self.b_conv.dtype != self.w_conv.dtype:
+            self.w_conv, self.b_conv = self.w_conv.float(), self.b_conv.float()
+        self.dt_bias, self.a_log, self.skip = (t(n).float().contiguous() for n in ("dt_bias", "A_log", "D"))
+        self.w_norm, self.w_o = t("norm").contiguous(), t("o")
+
+    def state_need(self):
+        needs = [StateNeed((self.n_heads, self.state_dim, self.value_dim), torch.float32, 0.0)]
+        if self.taps > 1:
+            needs.append(StateNeed((self.taps - 1, self.conv_cols), self.rt.act_dtype, 0.0))
+        return tuple(needs)
+
+    def products(self):
+        up16 = lambda n: n + (-n % 16)
+        return ((up16(self.main_rows), self.hidden), (up16(self.n_heads), self.hidden), (self.hidden, self.inner))
+
+    def forward(self, h: torch.Tensor, ctx, site) -> torch.Tensor:
+        ops, act = self.rt.ops, self.rt.act_dtype
+        proj = ops.linear(h, self.w_main, act)
+        dt = ops.linear(h, self.w_dt, torch.float32)  # the steps' logits per head, float32
+        xbc = proj[:, self.inner: self.inner + self.conv_cols]
+        conv_state = site.state(1) if self.taps > 1 else None
+        u = ops.causal_conv(xbc, self.w_conv, self.b_conv, conv_state, ctx, act="silu")
+        if conv_state is not None:
+            ops.conv_state_push(xbc, conv_state, ctx)
+        o = ops.linear_state_scan(
+            u, self.n_heads, self.groups, self.state_dim, self.value_dim, site.state(0), ctx, q_scale=1.0, unit_eps=None,
+            decay=("head", dt, 0, self.a_log, self.dt_bias), beta="step",
+            columns=(self.inner + self.bc_cols, self.inner, 0), skip=self.skip,
+        )
+        y = ops.gated_head_norm(o, self.w_norm, self.out_eps, proj, 0, self.norm_groups, self.inner // self.norm_groups, act,
+                                gate_first=True)
+        return ops.linear(y, self.w_o, act, partial_ok=True)

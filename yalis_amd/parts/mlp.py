@@ -6,7 +6,8 @@ biases.  The reference keeps gate and up in one matrix with rows interleaved (:7
 its products want, which is the same arithmetic.  The activation and product are computed
 in float32 on the projection's output.
 
-params: prefix, hidden_size, intermediate_size, activation ("silu"), names
+params: prefix, hidden_size, intermediate_size, activation ("silu", "gelu_tanh", or a gated pair with
+constants as the kernel library names them: ("clamped_swish", limit, slope)), names
 (optional overrides of the three tensor names below the prefix), bias (False; True: the
 three projections have biases ``*.bias`` beside their weights, which Llama's do not).
 """
@@ -33,8 +34,12 @@ class GatedMLP(FeedForward):
         self.hidden = int(params["hidden_size"])
         self.inter = int(params["intermediate_size"])
         self.activation = params.get("activation", "silu")
-        if self.activation not in ACTIVATIONS:
-            raise ValueError(f"activation {self.activation!r} is not supported (supported: {ACTIVATIONS})")
+        if isinstance(self.activation, str):
+            if self.activation not in ACTIVATIONS:
+                raise ValueError(f"activation {self.activation!r} is not supported (supported: {ACTIVATIONS})")
+        else:  # a gated pair with constants, (name, constants...): whatever the kernel library knows
+            self.activation = tuple(self.activation)
+            rt.ops.gated_kind(self.activation)
         names = {"gate": "gate_proj.weight", "up": "up_proj.weight", "down": "down_proj.weight"}
         names.update(params.get("names", {}))
         self.names = {k: f"{self.prefix}.{v}" for k, v in names.items()}

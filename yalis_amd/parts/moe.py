@@ -100,3 +100,97 @@ class TableMoE(FeedForward):
             a = ops.gate_up_act(h, self.shared_gate_up, self.shared_group, self.shared["activation"], self.rt.act_dtype)
             dense = ops.linear(a, self.shared_down, self.rt.act_dtype, partial_ok=True)
         return ExpertRows(dense, rows, self.top, 1.0 / self.top)
+
+
+@register_feed_forward("routed_moe")
+class RoutedMoE(FeedForward):
+    """A mixture whose experts a learned router chooses: logits z = W_router h in float32, scores s = sigmoid(z), the
+    ``top`` experts with the largest scores; a chosen expert reads the token's input multiplied by its score (the
+    score weighs what goes in, not what comes out; scores are not renormalised) and the outputs are summed.  An
+    optional shared expert of the same form and a width of its own runs for every token and is added.  Experts
+    are gated feed-forwards without biases, down(act(gate x) * (up x)).
+
+    The router's product is a library product with float32 output; one kernel chooses and writes every token's row
+    once per chosen expert, scaled (``ops.moe_router_topk``); the experts' two products are the grouped ones of
+    ``ops.moe_experts`` with the router's choice as their table; one kernel sums a token's rows and the shared
+    expert's output (``ops.moe_combine``).
+
+    params: prefix, hidden_size, experts, top, intermediate_size, activation ("silu"), shared (None or
+    {"intermediate_size", "activation"}), names (optional: "router", "expert" with {e} for the expert's number,
+    "shared", "gate", "up", "down")."""
+
+    graph_capturable = True
+
+    def __init__(self, params, rt: Runtime):
+        super().__init__(params, rt)
+        self.prefix = params["prefix"]
+        self.hidden = int(params["hidden_size"])
+        self.experts = int(params["experts"])
+        self.top = int(params["top"])
+        self.inter = int(params["intermediate_size"])
+        self.activation = params.get("activation", "silu")
+        if not 1 <= self.top <= self.experts:
+            raise ValueError(f"{self.prefix}: top={self.top} of {self.experts} experts")
+        rt.ops.gated_kind(self.activation)
+        self.shared = params.get("shared")
+        names = {"router": "router", "expert": "e{e}", "shared": "shared", "gate": "gate", "up": "up", "down": "down"}
+        names.update(params.get("names", {}))
+        self.names = names
+        self.router_rows = self.experts + (-self.experts % 16)
+        self.w_router = self.w_gate_up = self.w_down = None
+        self.shared_gate_up = self.shared_down = None
+        self.shared_group = 0
+
+    def _name(self, owner: str, which: str) -> str:
+        return f"{self.prefix}.{owner}.{self.names[which]}"
+
+    def _expert(self, e: int) -> str:
+        return self.names["expert"].format(e=e)
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        # (random routers are made wide enough that tokens differ in what they choose)
+        specs = {f"{self.prefix}.{self.names['router']}": TensorSpec((self.experts, self.hidden), "float", ("normal", 0.5))}
+        for e in range(self.experts):
+            specs[self._name(self._expert(e), "gate")] = TensorSpec((self.inter, self.hidden))
+            specs[self._name(self._expert(e), "up")] = TensorSpec((self.inter, self.hidden))
+            specs[self._name(self._expert(e), "down")] = TensorSpec((self.hidden, self.inter))
+        if self.shared:
+            ff = int(self.shared["intermediate_size"])
+            specs[self._name(self.names["shared"], "gate")] = TensorSpec((ff, self.hidden))
+            specs[self._name(self.names["shared"], "up")] = TensorSpec((ff, self.hidden))
+            specs[self._name(self.names["shared"], "down")] = TensorSpec((self.hidden, ff))
+        return specs
+
+    def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
+        router = tensors[f"{self.prefix}.{self.names['router']}"]
+        pad = self.router_rows - self.experts
+        if pad:
+            router = torch.cat([router, torch.zeros((pad, self.hidden), dtype=router.dtype, device=router.device)], dim=0)
+        self.w_router = router.contiguous()
+        self.w_gate_up = torch.stack([
+            torch.stack([tensors[self._name(self._expert(e), "gate")], tensors[self._name(self._expert(e), "up")]])
+            for e in range(self.experts)
+        ]).contiguous()
+        self.w_down = torch.stack([tensors[self._name(self._expert(e), "down")] for e in range(self.experts)]).contiguous()
+        if self.shared:
+            s = self.names["shared"]
+            self.shared_gate_up, self.shared_group = self.rt.ops.pack_gate_up(tensors[self._name(s, "gate")], tensors[self._name(s, "up")])
+            self.shared_down = tensors[self._name(s, "down")]
+
+    def products(self):
+        out = [(self.router_rows, self.hidden)]
+        if self.shared:
+            ff = int(self.shared["intermediate_size"])
+            out += [(2 * ff, self.hidden), (self.hidden, ff)]
+        return tuple(out)
+
+    def forward(self, h: torch.Tensor, ctx):
+        ops = self.rt.ops
+        logits = ops.linear(h, self.w_router, torch.float32)
+        choice, scaled = ops.moe_router_topk(logits, h, self.top, experts=self.experts)
+        rows = ops.moe_experts(scaled, None, choice, self.w_gate_up, self.w_down, self.activation)
+        dense = None
+        if self.shared:
+            a = ops.gate_up_act(h, self.shared_gate_up, self.shared_group, self.shared.get("activation", "silu"), self.rt.act_dtype)
+            dense = ops.linear(a, self.shared_down, self.rt.act_dtype, partial_ok=True)
+        return ops.moe_combine(dense, rows, self.top, 1.0)
