@@ -30,6 +30,11 @@ def embedding(W, tokens):
     return W["embed"][torch.tensor(tokens)] + W["pos"][:n]
 
 
+# when a list: for every query and head of every attention (both kinds), (query, head, the key with the largest
+# weight, that weight) is appended (tests that make attention sharp look where it points)
+ATTENTION_PEAKS: Optional[list] = None
+
+
 def latent_attention(W, p: str, m: dict, eps: float, h):
     n, H, d, vd = h.shape[0], m["heads"], m["dim"], m["vdim"]
     c_q = rms(h @ W[p + "dq"].T, eps) * W[p + "dq.norm"]
@@ -45,6 +50,8 @@ def latent_attention(W, p: str, m: dict, eps: float, h):
             e = torch.exp(s - top)
             den = e.sum() + math.exp(float(W[p + "sink"][hd]) - top)
             out[i, hd] = (e / den) @ v[: i + 1, hd]
+            if ATTENTION_PEAKS is not None:
+                ATTENTION_PEAKS.append((i, hd, int(torch.argmax(e)), float((e / den).max())))
     gate = torch.sigmoid(h @ W[p + "g"].T)
     return (out.reshape(n, H * vd) * gate) @ W[p + "o"].T
 
@@ -70,7 +77,10 @@ def window_attention(W, p: str, m: dict, h):
             g = hd // (H // G)
             s = (k[first: i + 1, g] @ q[i, hd]) * m["scale"]
             s = s + torch.stack([rel[distance_bucket(i - j, rel.shape[0], m["bias_max"]), hd] for j in range(first, i + 1)])
-            out[i, hd] = torch.softmax(s, 0) @ v[first: i + 1, g]
+            w = torch.softmax(s, 0)
+            out[i, hd] = w @ v[first: i + 1, g]
+            if ATTENTION_PEAKS is not None:
+                ATTENTION_PEAKS.append((i, hd, first + int(torch.argmax(w)), float(w.max())))
     gate = torch.sigmoid(h @ W[p + "g"].T)
     return (out.reshape(n, H * vd) * gate) @ W[p + "o"].T
 
@@ -118,12 +128,22 @@ def silu_expert(W, p: str, h):
     return ((g * torch.sigmoid(g)) * (h @ W[p + "up"].T)) @ W[p + "down"].T
 
 
+# when a list: every token's gap between the last chosen expert's logit and the best one left out is appended
+# (tests pick weights for which no choice is a close call)
+ROUTER_GAPS: Optional[list] = None
+
+
 def moe_ff(W, p: str, f: dict, h):
     n = h.shape[0]
-    scores = torch.sigmoid(h @ W[p + "router"].T)
+    logits = h @ W[p + "router"].T
+    scores = torch.sigmoid(logits)
     out = torch.zeros(n, W[p + "e0.down"].shape[0], dtype=F)
+    top = f["router"]["top"]
     for t in range(n):
-        chosen = torch.topk(scores[t], f["router"]["top"]).indices.tolist()
+        chosen = torch.topk(scores[t], top).indices.tolist()
+        if ROUTER_GAPS is not None and top < logits.shape[1]:
+            ranked = torch.sort(logits[t], descending=True).values
+            ROUTER_GAPS.append(float(ranked[top - 1] - ranked[top]))
         for e in chosen:
             out[t] += silu_expert(W, f"{p}e{e}.", (scores[t, e] * h[t])[None])[0]
     if f.get("shared"):
