@@ -32,6 +32,10 @@ kernel library, its bound max(bytes / 8 TB/s, flops / 2.5 PFLOP/s) and time / bo
 ``--design nutavik`` does the same for the Nutavik design (latent attention, delta rule, gated linear
 attention, dense feed-forward) beside the Llama configuration of equal width, depth, heads and
 feed-forward weights.
+``--design mesolix`` measures the Mesolix design (latent attention with sinks, state space duality, windowed
+attention with a bias per distance, dense and routed feed-forwards) beside the Nutavik configuration of equal width,
+depth, heads, latent and feed-forward sizes (the closest of the engine's models: latent attention and matrix-state
+recurrences) and the Llama configuration of equal size.
 """
 import argparse
 import json
@@ -408,6 +412,8 @@ def _op_costs(ops, hb):
     def moe(a, kw, out):
         x, table, wgu, wd = a[0], a[2], a[3], a[4]
         m, top, experts = x.shape[0], table.shape[1], wgu.shape[0]
+        if a[1] is None:  # a router's choice: the input has a row per (token, chosen expert) already
+            m //= top
         per_expert = wgu[0].numel() + wd[0].numel()
         return 2.0 * m * top * per_expert, 2.0 * min(m * top, experts) * per_expert + nbytes(x) * (1 + top) + 4.0 * m * top * x.shape[1]
 
@@ -449,7 +455,8 @@ def _op_costs(ops, hb):
             "rglru": rglru, "norm_add": moved, "add_rmsnorm": moved, "gather_add_rmsnorm": moved, "qkv_prepare": moved,
             "rope_append": moved, "causal_conv": moved, "gated_act": moved, "round_rows": moved, "embed": moved,
             "sandwich_norm": moved, "activation": moved, "latent_prepare": moved, "head_linear": head_linear,
-            "latent_attention": latent_attention, "linear_state_scan": state_scan, "gated_head_norm": moved, "conv_state_push": moved}
+            "latent_attention": latent_attention, "linear_state_scan": state_scan, "gated_head_norm": moved, "conv_state_push": moved, "moe_router_topk": moved,
+            "moe_combine": moved, "attention_finish": moved}
 
 
 def per_op_times(runner, vocab: int, gen, batch: int, prompt_len: int, prefill_len: int):
@@ -539,16 +546,20 @@ def design_compare(args) -> int:
     the Llama configuration of equal size; one JSON line a size."""
     import torch
 
-    from yalis_amd.models.presets import llama_like
+    from yalis_amd.models.presets import llama_like, nutavik_like
 
-    sizes = {"suranex": ("suranex-2k", "suranex-4k"), "nutavik": ("nutavik-2k", "nutavik-4k")}[args.design]
+    sizes = {"suranex": ("suranex-2k", "suranex-4k"), "nutavik": ("nutavik-2k", "nutavik-4k"), "mesolix": ("mesolix-2k", "mesolix-4k")}[args.design]
     if args.design_shape:
         sizes = (args.design_shape,)
     for name in sizes:
         label, cfg = SHAPES[name]
         line = {"design": args.design, "shape": label, "batch": args.batch, "prompt_len": args.prompt_len, "prefill_len": args.prefill_len,
                 "dtype": "bf16", "data": "synthetic: random bf16 weights, seeded uniform-random token ids"}
-        for who, c in (("design", cfg), ("llama_of_equal_size", llama_like(cfg))):
+        beside = [("design", cfg)]
+        if args.design == "mesolix":
+            beside.append(("nutavik_of_equal_size", nutavik_like(cfg)))
+        beside.append(("llama_of_equal_size", llama_like(cfg)))
+        for who, c in beside:
             gen = torch.Generator().manual_seed(0)
             vocab = c.get("vocab", c.get("vocab_size"))
             steps = args.steps
@@ -570,9 +581,9 @@ def design_compare(args) -> int:
 
 def main() -> int:
     ap = argparse.ArgumentParser()
-    ap.add_argument("--design", choices=("suranex", "nutavik"), default=None,
+    ap.add_argument("--design", choices=("suranex", "nutavik", "mesolix"), default=None,
                     help="measure instead another design's prefill and decode at a few layer sizes, beside the Llama configuration of equal size, with the time and the bound of every kind of kernel")
-    ap.add_argument("--design-shape", default=None, help="with --design: one of its shapes only (suranex-2k, suranex-4k, nutavik-2k, nutavik-4k)")
+    ap.add_argument("--design-shape", default=None, help="with --design: one of its shapes only (suranex-2k, suranex-4k, nutavik-2k, nutavik-4k, mesolix-2k, mesolix-4k)")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=32)
     ap.add_argument("--warmup", type=int, default=4)

@@ -130,7 +130,9 @@ extern "C" int yk_attn_generic(const void* q, int q_stride, void* out, const voi
 // ------------------------------------------------------------------------ matrix cores
 // Options of the matrix-core kernels beyond the plain causal window (their EXT instantiations; the
 // plain ones are compiled without): the first `keep_first` keys of a request stay visible below
-// the window, and a score s (times the scale) is squashed to cap * tanh(s / cap).
+// the window, a score s (times the scale) is squashed to cap * tanh(s / cap), and a learned bias per head
+// and distance (a float32 table [distances][heads], the last row for everything farther) is added to
+// the scaled, squashed score.
 //
 // Kept first keys add blocks of 64 keys in front of the window's: a kernel numbers the blocks it
 // walks "virtually", the window's blocks by their own number and the n_first blocks of kept keys
@@ -146,6 +148,12 @@ __device__ __forceinline__ int ext_block(int vb, int first_window_block, int n_f
 __device__ __forceinline__ float ext_squash(float s, float cap_over_scale, float scale_over_cap_2log2e) {
   const float e = __builtin_amdgcn_exp2f(s * scale_over_cap_2log2e);  // e^(2x); inf and 0 at the ends give +-1
   return cap_over_scale * (1.f - __fdividef(2.f, 1.f + e));
+}
+
+// a learned bias per head and distance: row min(n, rows - 1) of a float32 table [rows][heads] whose column `col`
+// points at (a key ahead of the query, which the mask drops anyway, reads row 0)
+__device__ __forceinline__ float ext_bias(const float* __restrict__ col, int n, int rows, int n_heads) {
+  return col[static_cast<size_t>(min(max(n, 0), rows - 1)) * n_heads];
 }
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
@@ -249,7 +257,8 @@ __global__ __launch_bounds__(64 * W, 2) void attn_mfma_kernel(
     const int32_t* __restrict__ tiles, const int32_t* __restrict__ block_table, int table_width,
     int page_size, int n_heads, int n_kv, int hpt, int chunks, float scale_log2, int window,
     int n_splits, float* __restrict__ ws_o, float* __restrict__ ws_ml, RopeSrc rs, int keep_first_arg = 0,
-    float cap_over_scale = 0.f, float scale_over_cap_2log2e = 0.f) {
+    float cap_over_scale = 0.f, float scale_over_cap_2log2e = 0.f, const float* __restrict__ dist_bias = nullptr,
+    int bias_rows = 0, float inv_scale = 0.f) {
   const int keep_first = EXT ? keep_first_arg : 0;
   constexpr int KS = D / 32;  // matrix-core steps over the head dimension
   constexpr int DT = D / 16;  // output tiles over the head dimension
@@ -535,6 +544,17 @@ __global__ __launch_bounds__(64 * W, 2) void attn_mfma_kernel(
 #pragma unroll
           for (int i = 0; i < 4; ++i) s[u][sb][i] = ext_squash(s[u][sb][i], cap_over_scale, scale_over_cap_2log2e);
     }
+    if (EXT && dist_bias != nullptr) {
+      // the column's head's bias for the key's distance, in the raw score's units (the scale multiplies later)
+      const float* bcol = dist_bias + h_base + min(hh, heads_here - 1);
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int sb = 0; sb < 2; ++sb)
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            s[u][sb][i] = fmaf(ext_bias(bcol, pos_c - (akb * 64 + 32 * u + 8 * gq + 4 * sb + i), bias_rows, n_heads), inv_scale, s[u][sb][i]);
+    }
 #pragma unroll
     for (int u = 0; u < 2; ++u)
 #pragma unroll
@@ -696,7 +716,7 @@ __global__ __launch_bounds__(256, CT == 1 ? 3 : 2) void attn_mfma_prefill_kernel
     const int32_t* __restrict__ tiles, const int32_t* __restrict__ block_table, int table_width,
     int page_size, int n_heads, int n_kv, int hpt, int chunks, float scale_log2, int window,
     int n_splits, float* __restrict__ ws_o, float* __restrict__ ws_ml, int pages_lds_limit, int keep_first_arg,
-    float cap_over_scale, float scale_over_cap_2log2e) {
+    float cap_over_scale, float scale_over_cap_2log2e, const float* __restrict__ dist_bias, int bias_rows, float inv_scale) {
   constexpr int KS = D / 32, DT = D / 16;
   const int keep_first = EXT ? keep_first_arg : 0;
   constexpr int KROW = D + 8;   // bf16 elements per parked key row
@@ -907,6 +927,19 @@ __global__ __launch_bounds__(256, CT == 1 ? 3 : 2) void attn_mfma_prefill_kernel
 #pragma unroll
             for (int i = 0; i < 4; ++i) s[c][u][sb][i] = ext_squash(s[c][u][sb][i], cap_over_scale, scale_over_cap_2log2e);
     }
+    if (EXT && dist_bias != nullptr) {
+      // the column's head's bias for the key's distance, in the raw score's units (the scale multiplies later)
+      const float* bcol = dist_bias + h_base + min(hh, heads_here - 1);
+#pragma unroll
+      for (int c = 0; c < CT; ++c)
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+          for (int sb = 0; sb < 2; ++sb)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+              s[c][u][sb][i] = fmaf(ext_bias(bcol, pos_c[c] - (key0 + 32 * u + 8 * gq + 4 * sb + i), bias_rows, n_heads), inv_scale, s[c][u][sb][i]);
+    }
     AFrag8 pf[CT][2];
     float alpha[CT];
     bool grew = false;  // some column's maximum rose: only then the running sums need rescaling
@@ -1068,7 +1101,8 @@ extern "C" int yk_attn_mfma_prefill(const void* q, int q_stride, void* out, cons
                                     const int32_t* block_table, int table_width, int page_size,
                                     int head_dim, int n_heads, int n_kv, float scale, int window,
                                     int n_splits, int col_tiles, float* workspace, size_t workspace_floats,
-                                    int pages_lds_limit, int keep_first, float softcap, hipStream_t stream) {
+                                    int pages_lds_limit, int keep_first, float softcap, const float* dist_bias, int bias_rows,
+                                    hipStream_t stream) {
   YK_REQUIRE(n_tiles >= 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0, "attn_mfma_prefill: bad head counts");
   YK_REQUIRE(col_tiles == 1 || col_tiles == 2, "attn_mfma_prefill: a wave has 1 or 2 column tiles");
   YK_REQUIRE(yk_attn_mfma_supported(head_dim), "attn_mfma_prefill: head_dim must be 64 or 128");
@@ -1080,8 +1114,10 @@ extern "C" int yk_attn_mfma_prefill(const void* q, int q_stride, void* out, cons
   YK_REQUIRE(window >= 0 && table_width > 0, "attn_mfma_prefill: bad window or table");
   YK_REQUIRE(scale > 0.f, "attn_mfma_prefill: the score scale must be positive");
   YK_REQUIRE(keep_first >= 0 && softcap >= 0.f, "attn_mfma_prefill: keep_first and softcap must not be negative");
+  YK_REQUIRE(dist_bias == nullptr || bias_rows >= 1, "attn_mfma_prefill: an empty table of biases");
   if (n_tiles == 0) return 0;
-  const bool ext = (keep_first > 0 && window > 0) || softcap > 0.f;
+  const bool ext = (keep_first > 0 && window > 0) || softcap > 0.f || dist_bias != nullptr;
+  const float inv_scale = 1.f / scale;
   const float cap_over_scale = softcap > 0.f ? softcap / scale : 0.f;
   const float scale_over_cap = softcap > 0.f ? scale / softcap * 2.f * 1.4426950408889634f : 0.f;
   const int hpt = yk_attn_heads_per_tile(n_heads, n_kv);
@@ -1097,7 +1133,8 @@ extern "C" int yk_attn_mfma_prefill(const void* q, int q_stride, void* out, cons
 #define YK_PF_ARGS                                                                                           \
   static_cast<const bf16_t*>(q), q_stride, static_cast<bf16_t*>(out), static_cast<const bf16_t*>(k_cache),     \
       static_cast<const bf16_t*>(v_cache), tiles, block_table, table_width, page_size, n_heads, n_kv, hpt,     \
-      chunks, scale_log2, window, n_splits, ws_o, ws_ml, pages_lds_limit, keep_first, cap_over_scale, scale_over_cap
+      chunks, scale_log2, window, n_splits, ws_o, ws_ml, pages_lds_limit, keep_first, cap_over_scale, scale_over_cap, \
+      dist_bias, bias_rows, inv_scale
 #define YK_PF(DD, BIP)                                                                                       \
   if (ext && col_tiles == 2)                                                                                 \
     attn_mfma_prefill_kernel<DD, BIP, 2, true><<<grid, block, 0, stream>>>(YK_PF_ARGS);                      \
@@ -1136,10 +1173,12 @@ static int launch_attn_mfma(const void* q, int q_stride, void* out, const void* 
                             int page_size, int head_dim, int n_heads, int n_kv, float scale, int window,
                             int n_waves, int n_splits, float* workspace, size_t workspace_floats,
                             int leave_splits, const RopeSrc* rope, bool rope_f32, hipStream_t stream, int keep_first = 0,
-                            float softcap = 0.f) {
+                            float softcap = 0.f, const float* dist_bias = nullptr, int bias_rows = 0) {
   YK_REQUIRE(n_tiles >= 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0, "attn_mfma: bad head counts");
   YK_REQUIRE(keep_first >= 0 && softcap >= 0.f, "attn_mfma: keep_first and softcap must not be negative");
-  const bool ext = (keep_first > 0 && window > 0) || softcap > 0.f;
+  YK_REQUIRE(dist_bias == nullptr || bias_rows >= 1, "attn_mfma: an empty table of biases");
+  const bool ext = (keep_first > 0 && window > 0) || softcap > 0.f || dist_bias != nullptr;
+  const float inv_scale = scale > 0.f ? 1.f / scale : 0.f;
   YK_REQUIRE(!(ext && rope), "attn_mfma: kept first keys and squashed scores are not offered with rotary inside the launch");
   const float cap_over_scale = softcap > 0.f ? softcap / scale : 0.f;
   const float scale_over_cap = softcap > 0.f ? scale / softcap * 2.f * 1.4426950408889634f : 0.f;
@@ -1179,11 +1218,11 @@ static int launch_attn_mfma(const void* q, int q_stride, void* out, const void* 
   }
 #define YK_LAUNCH_EXT(DD)                                                                          \
   if (tiled) {                                                                                     \
-    if (n_waves == 1) attn_mfma_kernel<DD, 1, true, 0, true><<<grid, block, 0, stream>>>(YK_ARGS, keep_first, cap_over_scale, scale_over_cap); \
-    else attn_mfma_kernel<DD, 4, true, 0, true><<<grid, block, 0, stream>>>(YK_ARGS, keep_first, cap_over_scale, scale_over_cap); \
+    if (n_waves == 1) attn_mfma_kernel<DD, 1, true, 0, true><<<grid, block, 0, stream>>>(YK_ARGS, keep_first, cap_over_scale, scale_over_cap, dist_bias, bias_rows, inv_scale); \
+    else attn_mfma_kernel<DD, 4, true, 0, true><<<grid, block, 0, stream>>>(YK_ARGS, keep_first, cap_over_scale, scale_over_cap, dist_bias, bias_rows, inv_scale); \
   } else {                                                                                         \
-    if (n_waves == 1) attn_mfma_kernel<DD, 1, false, 0, true><<<grid, block, 0, stream>>>(YK_ARGS, keep_first, cap_over_scale, scale_over_cap); \
-    else attn_mfma_kernel<DD, 4, false, 0, true><<<grid, block, 0, stream>>>(YK_ARGS, keep_first, cap_over_scale, scale_over_cap); \
+    if (n_waves == 1) attn_mfma_kernel<DD, 1, false, 0, true><<<grid, block, 0, stream>>>(YK_ARGS, keep_first, cap_over_scale, scale_over_cap, dist_bias, bias_rows, inv_scale); \
+    else attn_mfma_kernel<DD, 4, false, 0, true><<<grid, block, 0, stream>>>(YK_ARGS, keep_first, cap_over_scale, scale_over_cap, dist_bias, bias_rows, inv_scale); \
   }
 #define YK_LAUNCH(DD)                                                                              \
   if (ext) { YK_LAUNCH_EXT(DD) } else                                                              \
@@ -1211,10 +1250,11 @@ extern "C" int yk_attn_mfma(const void* q, int q_stride, void* out, const void* 
                             const int32_t* block_table, int table_width, int page_size,
                             int head_dim, int n_heads, int n_kv, float scale, int window,
                             int n_waves, int n_splits, float* workspace, size_t workspace_floats,
-                            int leave_splits, int keep_first, float softcap, hipStream_t stream) {
+                            int leave_splits, int keep_first, float softcap, const float* dist_bias, int bias_rows,
+                            hipStream_t stream) {
   return launch_attn_mfma(q, q_stride, out, k_cache, v_cache, tiles, n_tiles, block_table, table_width, page_size,
                           head_dim, n_heads, n_kv, scale, window, n_waves, n_splits, workspace, workspace_floats,
-                          leave_splits, nullptr, false, stream, keep_first, softcap);
+                          leave_splits, nullptr, false, stream, keep_first, softcap, dist_bias, bias_rows);
 }
 
 // yk_attn_mfma for a step of single tokens (every tile holds ONE token), with rotary + append

@@ -80,12 +80,45 @@ def nutavik_shape(width: int, vocab: int, heads: int, dim: int, rot_dim: int, kv
             "layers": layers}
 
 
+def mesolix_shape(width: int, vocab: int, heads: int, kv_heads: int, dim: int, kv_rank: int, q_rank: int, window: int, ssd_heads: int,
+                  ssd_vdim: int, state: int, groups: int, ff: int, experts: int, top: int, expert_ff: int, shared_ff: int,
+                  bias_rows: int = 32, max_positions: int = 8192, repeats: int = 2, again: bool = False) -> dict:
+    """A Mesolix config.json of the given layer sizes: (latent attention, state space duality, windowed attention
+    with a bias per distance) repeated ``repeats`` times, dense and routed feed-forwards in turn; with ``again`` a last
+    layer runs the first one's weights once more."""
+    lat = {"heads": heads, "dim": dim, "vdim": dim, "kv_rank": kv_rank, "q_rank": q_rank, "scale": dim ** -0.5}
+    ssd = {"heads": ssd_heads, "vdim": ssd_vdim, "state": state, "groups": groups, "conv": 4, "norm_groups": groups}
+    att = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5, "bias_max": float(2 * window),
+           "bias_rows": bias_rows, "mask": {"size": window}}
+    dense = {"kind": "dense", "ff": ff, "limit": 7.0}
+    moe = {"kind": "moe", "router": {"experts": experts, "top": top}, "expert": {"ff": expert_ff}, "shared": {"ff": shared_ff}}
+    layers = []
+    for r in range(repeats):
+        for i, (kind, mixer) in enumerate((("latent_attention", lat), ("mamba2", ssd), ("attention", att))):
+            layers.append({"type": kind, "mixer": dict(mixer), "mlp": dict(dense if (3 * r + i) % 2 == 0 else moe)})
+    if again:
+        layers.append(dict(layers[0], weights_of=0))
+    return {"architecture": "Mesolix", "vocab": vocab, "width": width, "max_positions": max_positions, "norm": {"eps": 1e-6}, "layers": layers}
+
+
 def llama_like(design: dict) -> dict:
     """The Llama configuration of equal size.  For Suranex: the same width, layer count, vocabulary
     and (first attention layer's) heads, a feed-forward as wide as what a token uses of the mixture
     (its top experts and the shared one).  For Nutavik: the same width, layer count, vocabulary and
     attention heads (keys as wide as its unrotated and rotated parts together, a quarter as many key
     heads), a gated feed-forward with as many weights as its dense one (two thirds as wide)."""
+    if design.get("architecture") == "Mesolix":
+        # the same width, layer count, vocabulary and (windowed attention's) heads; a feed-forward with as many
+        # weights as the mean of what a token uses of the dense and the routed ones
+        att = next(layer["mixer"] for layer in design["layers"] if layer["type"] == "attention")
+        used = []
+        for layer in design["layers"]:
+            f = layer["mlp"]
+            if f is not None:
+                used.append(f["ff"] if f["kind"] == "dense" else f["router"]["top"] * f["expert"]["ff"] + (f["shared"]["ff"] if f.get("shared") else 0))
+        inter = (sum(used) // max(len(used), 1) + 255) // 256 * 256
+        return dict(LLAMA3_8B, hidden_size=design["width"], num_hidden_layers=len(design["layers"]), num_attention_heads=att["heads"],
+                    num_key_value_heads=att["kv_heads"], head_dim=att["dim"], intermediate_size=inter, vocab_size=design["vocab"])
     if design.get("architecture") == "Nutavik":
         att = next(layer["mixer"] for layer in design["layers"] if layer["type"] == "latent_attention")
         ff = next(layer["mlp"]["ff"] for layer in design["layers"] if layer["mlp"] is not None)
@@ -101,12 +134,28 @@ def llama_like(design: dict) -> dict:
                 num_key_value_heads=att["kv_heads"], head_dim=att["dim"], intermediate_size=inter, vocab_size=suranex["vocab"])
 
 
+def nutavik_like(design: dict) -> dict:
+    """The Nutavik configuration of a Mesolix one's size: the same width, vocabulary and layer count (in threes), a
+    latent attention of the same heads and ranks with a rotated part of 64 (or a quarter of the latent) on top, the
+    two recurrences with as many heads and as wide keys and values as the state-space layer's state and channels,
+    a dense feed-forward as wide as Mesolix's dense one."""
+    lat = next(layer["mixer"] for layer in design["layers"] if layer["type"] == "latent_attention")
+    ssd = next(layer["mixer"] for layer in design["layers"] if layer["type"] == "mamba2")
+    ff = next(layer["mlp"]["ff"] for layer in design["layers"] if layer["mlp"] is not None and layer["mlp"]["kind"] == "dense")
+    rot = 64 if lat["kv_rank"] >= 256 else max(2, lat["kv_rank"] // 4)
+    return nutavik_shape(design["width"], design["vocab"], lat["heads"], lat["dim"], rot, lat["kv_rank"], lat["q_rank"], ssd["heads"],
+                         max(1, ssd["heads"] // 2), ssd["heads"], ssd["state"], ssd["vdim"], ff, repeats=max(1, len(design["layers"]) // 3))
+
+
 SURANEX_2K = suranex_shape(2048, 32768, 16, 4, 128, 1024, 2560, 10, 16, 2, 1024, 2048)
 SURANEX_4K = suranex_shape(4096, 65536, 32, 8, 128, 2048, 5120, 20, 32, 4, 1024, 4096, repeats=1)
 SURANEX_TINY = suranex_shape(64, 256, 4, 2, 16, 24, 96, 3, 4, 2, 32, 48, repeats=1)
 NUTAVIK_2K = nutavik_shape(2048, 32768, 16, 128, 64, 512, 768, 16, 8, 4, 256, 512, 8192)
 NUTAVIK_4K = nutavik_shape(4096, 65536, 32, 128, 64, 512, 1536, 32, 16, 8, 256, 512, 16384, repeats=1)
 NUTAVIK_TINY = nutavik_shape(64, 256, 4, 16, 8, 24, 32, 4, 2, 2, 16, 32, 96, repeats=1)
+MESOLIX_2K = mesolix_shape(2048, 32768, 16, 4, 128, 512, 768, 1024, 32, 64, 128, 2, 8192, 16, 2, 1024, 2048)
+MESOLIX_4K = mesolix_shape(4096, 65536, 32, 8, 128, 512, 1536, 2048, 64, 64, 128, 4, 16384, 32, 4, 1024, 4096, repeats=1)
+MESOLIX_TINY = mesolix_shape(64, 256, 4, 2, 16, 24, 32, 24, 4, 8, 16, 2, 96, 4, 2, 32, 48, bias_rows=8, max_positions=256, repeats=1, again=True)
 
 # name -> (what to call it, config.json dictionary)
 SHAPES: Dict[str, Tuple[str, dict]] = {
@@ -122,6 +171,9 @@ SHAPES: Dict[str, Tuple[str, dict]] = {
     "nutavik-2k": ("Nutavik, width 2,048", NUTAVIK_2K),
     "nutavik-4k": ("Nutavik, width 4,096", NUTAVIK_4K),
     "nutavik-tiny": ("tiny Nutavik", NUTAVIK_TINY),
+    "mesolix-2k": ("Mesolix, width 2,048", MESOLIX_2K),
+    "mesolix-4k": ("Mesolix, width 4,096", MESOLIX_4K),
+    "mesolix-tiny": ("tiny Mesolix", MESOLIX_TINY),
 }
 
 

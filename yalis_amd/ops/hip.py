@@ -176,11 +176,11 @@ _SIGNATURES = {
     "yk_attn_tokens_per_tile": ([_c_int, _c_int], _c_int),
     "yk_attn_mfma_workspace": ([_c_int, _c_int, _c_int, _c_int, _c_int], _c_size_t),
     "yk_attn_mfma_prefill": (
-        [_vp, _c_int, _vp, _vp, _vp, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_int, _vp, _c_size_t, _c_int, _c_int, _c_float, _vp],
+        [_vp, _c_int, _vp, _vp, _vp, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_int, _vp, _c_size_t, _c_int, _c_int, _c_float, _vp, _c_int, _vp],
         _c_int,
     ),
     "yk_attn_mfma": (
-        [_vp, _c_int, _vp, _vp, _vp, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_int, _vp, _c_size_t, _c_int, _c_int, _c_float, _vp],
+        [_vp, _c_int, _vp, _vp, _vp, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_int, _vp, _c_size_t, _c_int, _c_int, _c_float, _vp, _c_int, _vp],
         _c_int,
     ),
     "yk_attn_mfma_rope": (
@@ -209,7 +209,7 @@ _LATER_SIGNATURES = {
         "yk_probe_mfma_bf16": ([_c_int, _c_int, _vp, _vp], _c_int),
     },
 }
-_ABI = 19
+_ABI = 20
 
 # Rows of x up to which the hand-written matrix-core kernel runs a bfloat16 product;
 # above it the vendor library does.
@@ -912,7 +912,7 @@ class HipOps:
     def attention(self, qkv, n_heads, n_kv, head_dim, k_cache, v_cache, page_size,
                   scale, window, ctx, group, tiles, long_tiles=None, plan=None, long_plan=None,
                   long_col_tiles: int = 1, token_cols=None, rope: Optional["RopeInLaunch"] = None,
-                  keep_first: int = 0, softcap: float = 0.0):
+                  keep_first: int = 0, softcap: float = 0.0, distance_bias=None):
         """Queries are the first n_heads heads of each row of ``qkv`` (whatever follows
         them in the row is skipped); keys and values come from the cache through the
         block table of ``group``.  ``long_tiles`` hold up to
@@ -924,7 +924,8 @@ class HipOps:
 
         ``keep_first`` / ``softcap`` (matrix-core kernels only; other sizes are ``attention_masked``'s): with a
         window, the first ``keep_first`` keys of a request stay visible below it; scores times the scale
-        are squashed to softcap * tanh(s / softcap).
+        are squashed to softcap * tanh(s / softcap); ``distance_bias`` (float32 [distances, n_heads]): row
+        min(p - j, distances - 1) is added to head h's scaled (and squashed) score of key j for the query at p.
 
         ``rope`` (only where ``attention_can_rotate``, and only for steps whose spans are single
         tokens): ``qkv`` is then the projection's raw output (a tensor or a ``SplitSum``) and
@@ -948,8 +949,12 @@ class HipOps:
             and qkv.stride(0) % 8 == 0
             and qkv.data_ptr() % 16 == 0
         )
-        if (keep_first or softcap) and not use_mfma:
-            raise KernelError("attention: kept first keys and squashed scores outside the matrix-core kernels' sizes are attention_masked's")
+        if (keep_first or softcap or distance_bias is not None) and not use_mfma:
+            raise KernelError("attention: kept first keys, squashed scores and biases per distance outside the matrix-core kernels' sizes are attention_masked's")
+        if distance_bias is not None and (distance_bias.dtype != torch.float32 or distance_bias.dim() != 2 or not distance_bias.is_contiguous()
+                                          or distance_bias.shape[1] != n_heads or distance_bias.shape[0] < 1):
+            raise KernelError("attention: the distance bias is contiguous float32 [distances, heads]")
+        bias_rows = 0 if distance_bias is None else distance_bias.shape[0]
         if use_mfma and long_tiles is not None and long_tiles.shape[0] > 0:
             n_long = long_tiles.shape[0]
             hpt = self._ask("yk_attn_heads_per_tile", n_heads, n_kv)
@@ -963,7 +968,7 @@ class HipOps:
                     long_tiles.data_ptr(), n_long, bt.data_ptr(), bt.shape[1], page_size, head_dim,
                     n_heads, n_kv, float(scale), int(window), long_splits, int(long_col_tiles), _ptr(ws),
                     0 if ws is None else ws.numel(), int(self.long_span_pages_in_lds), int(keep_first), float(softcap),
-                    self._stream(),
+                    _ptr(distance_bias), bias_rows, self._stream(),
                 )
             )
         if use_mfma and tiles.shape[0] == 0:
@@ -982,7 +987,7 @@ class HipOps:
                     qkv.data_ptr(), qkv.stride(0), out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
                     tiles.data_ptr(), n_tiles, bt.data_ptr(), bt.shape[1], page_size, head_dim, n_heads, n_kv,
                     float(scale), int(window), waves, splits, _ptr(ws), 0 if ws is None else ws.numel(), int(leave),
-                    int(keep_first), float(softcap), self._stream(),
+                    int(keep_first), float(softcap), _ptr(distance_bias), bias_rows, self._stream(),
                 )
             )
             if leave:

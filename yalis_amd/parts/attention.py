@@ -107,9 +107,7 @@ class Attention(Mixer):
             # the matrix-core kernels take these options too, where they take the sizes (bfloat16, keys and
             # values of 64 or 128 elements alike); everything else runs on the general float32-arithmetic kernel
             can = getattr(rt.ops, "attention_can_rotate", None)
-            # (a bias per distance is the general kernel's alone)
-            self.on_matrix_cores = bool(can is not None and self.value_dim == self.head_dim and can(rt.act_dtype, self.head_dim) is True
-                                        and not self.distance_bias)
+            self.on_matrix_cores = bool(can is not None and self.value_dim == self.head_dim and can(rt.act_dtype, self.head_dim) is True)
             if self.on_matrix_cores:
                 self._tile_sizes(rt)
             return
@@ -294,6 +292,7 @@ class Attention(Mixer):
                 ctx.arrays[f"attention_tiles_{self.tokens_per_tile}_upto{self.long_tile}"],
                 ctx.arrays[f"attention_long_tiles_{self.long_tile_2 if col_tiles == 2 else self.long_tile}_{self.layout}"],
                 long_col_tiles=col_tiles, keep_first=self.keep_first if self.window else 0, softcap=self.softcap,
+                distance_bias=self.bias_by_distance,
             )
             if self.value_rotation is not None or self.gate_name:
                 ops.attention_finish(out, ctx.arrays["positions"], self.n_heads, self.value_dim, self.value_rotation,
