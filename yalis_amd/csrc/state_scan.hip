@@ -310,8 +310,15 @@ __global__ __launch_bounds__(256) void linear_state_scan_kernel(
     }
     __syncthreads();
     // the walk; a token's k, q and decays are read from LDS while the token before is worked on
+    // (the token's scalars come with them: read where they are used, each costs the single wave of a SIMD a
+    // round trip to LDS that nothing hides)
     float kn[kScanRows], qn[kScanRows], an[kScanRows];
+    float a_n = 1.f, v_n = 0.f, b_n = 1.f, kq_n = 0.f;
     auto fetch = [&](int t) {
+      if (decay_mode != 1) a_n = as[t];
+      v_n = vs[t * cols_per_block + col_local];
+      b_n = bs[t];
+      kq_n = kqs[t];
       const float4* kt = reinterpret_cast<const float4*>(ks + t * DS + sub * kScanRows);
       const float4* qt = reinterpret_cast<const float4*>(qs + t * DS + sub * kScanRows);
 #pragma unroll
@@ -342,11 +349,11 @@ __global__ __launch_bounds__(256) void linear_state_scan_kernel(
 #pragma unroll
         for (int r = 0; r < kScanRows; ++r) S[r] *= an[r];
       } else {
-        const float a = as[t];
+        const float a = a_n;
 #pragma unroll
         for (int r = 0; r < kScanRows; ++r) S[r] *= a;
       }
-      const float v_t = vs[t * cols_per_block + col_local], b_t = bs[t], kq_t = kqs[t];
+      const float v_t = v_n, b_t = b_n, kq_t = kq_n;
       if (t + 1 < nt) fetch(t + 1);
       // both sums over the decayed S at once: S^T k for the write, S^T q for the read-out, which sees the
       // token's own write through q . (k u^T) = u (k . q)
