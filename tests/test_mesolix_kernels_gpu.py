@@ -57,7 +57,7 @@ def biased_attention(q, k, v, positions, heads_per_kv, scale, window, bias):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("head_dim,value_dim,heads,kv", [(64, 64, 4, 2), (128, 128, 6, 1), (32, 48, 4, 4), (64, 32, 4, 2)])
+@pytest.mark.parametrize("head_dim,value_dim,heads,kv", [(64, 64, 4, 2), (128, 128, 6, 1), (32, 48, 4, 4), (64, 32, 4, 2), (64, 64, 2, 2)])
 @pytest.mark.parametrize("special,window,rows", [(400, 200, 200), (401, 200, 200), (399, 200, 37), (0, 0, 64), (63, 0, 700), (64, 0, 5), (127, 0, 128),
                                                   (128, 700, 1), (536, 64, 64), (537, 64, 30), (599, 1, 4)])
 def test_biased_attention_at_every_edge(dtype, head_dim, value_dim, heads, kv, special, window, rows):
