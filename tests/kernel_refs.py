@@ -13,17 +13,21 @@ import math
 import torch
 
 
-def embed(token_ids, table, positions=None, position_table=None):
+def embed(token_ids, table, positions=None, position_table=None, scale=1.0):
     x = table[token_ids.long()].to(torch.float32)
+    if scale != 1.0:
+        x = x * torch.tensor(scale, dtype=torch.float32)
     if position_table is not None:
         x = x + position_table[positions.long()].to(torch.float32)
     return x
 
 
-def add_rmsnorm(residual, delta, weight, eps, unit_offset, out_dtype):
-    """residual += delta in place (float32); returns the normalised rows."""
+def add_rmsnorm(residual, delta, weight, eps, unit_offset, out_dtype, row=None):
+    """residual += delta (+ row, one vector for every token) in place (float32); returns the normalised rows."""
     if delta is not None:
         residual += delta.to(torch.float32)
+    if row is not None:
+        residual += row.to(torch.float32)
     return _rmsnorm(residual, weight, eps, unit_offset).to(out_dtype)
 
 
@@ -297,18 +301,55 @@ def _turn(x, cos, sin, rot, interleaved, sign=1.0):
     return x
 
 
+def query_temperature(positions, coef, every):
+    """float32 1 + coef ln(floor((p + 1) / every) + 1)."""
+    steps = torch.div(positions.long() + 1, int(every), rounding_mode="floor").to(torch.float32)
+    return 1.0 + torch.tensor(coef, dtype=torch.float32) * torch.log(steps + 1.0)
+
+
+def qk_row_scales(proj, n_q_cols, n_k_cols, positions, bias=None, eps=None, temperature=None):
+    """float32 [N, 2]: what a token's queries (column 0) and keys (column 1) are multiplied with as wholes: with
+    ``eps`` the inverse root mean square over all the query columns (all the key columns) of the biased projection,
+    with ``temperature`` = (coef, every) the queries' factor by position on top."""
+    x = proj.to(torch.float32)
+    if bias is not None:
+        x = x + bias[: x.shape[1]]
+    out = torch.ones((x.shape[0], 2), dtype=torch.float32, device=x.device)
+    if eps is not None:
+        q, k = x[:, :n_q_cols], x[:, n_q_cols: n_q_cols + n_k_cols]
+        out[:, 0] = torch.rsqrt((q * q).mean(-1) + eps)
+        if n_k_cols:
+            out[:, 1] = torch.rsqrt((k * k).mean(-1) + eps)
+    if temperature is not None:
+        out[:, 0] = out[:, 0] * query_temperature(positions, *temperature)
+    return out
+
+
 def qkv_prepare(qkv, n_heads, n_kv, head_dim, value_dim, positions, act_dtype, q_norm=None, k_norm=None, qk_eps=0.0,
-                rotation=None, value_norm_eps=None, value_rotation=None, k_cache=None, v_cache=None, slots=None, page_size=0):
+                rotation=None, value_norm_eps=None, value_rotation=None, k_cache=None, v_cache=None, slots=None, page_size=0,
+                bias=None, row_scales=None, norm_over_projection=False, values_from_keys=False):
     n = qkv.shape[0]
     x = qkv.to(torch.float32)
+    if bias is not None:
+        x = x + bias[: x.shape[1]]
     hd = n_heads * head_dim
     q = x[:, :hd].reshape(n, n_heads, head_dim)
     k = x[:, hd: hd + n_kv * head_dim].reshape(n, n_kv, head_dim)
-    v = x[:, hd + n_kv * head_dim: hd + n_kv * (head_dim + value_dim)].reshape(n, n_kv, value_dim)
+    if values_from_keys:
+        v = k
+    else:
+        v = x[:, hd + n_kv * head_dim: hd + n_kv * (head_dim + value_dim)].reshape(n, n_kv, value_dim)
     pos = positions.long()
-    if q_norm is not None:
+    if norm_over_projection:  # the inverse root mean square comes with the row scales; the weights span the projection
+        q = q * q_norm.to(torch.float32).view(1, n_heads, head_dim)
+        if n_kv:
+            k = k * k_norm.to(torch.float32).view(1, n_kv, head_dim)
+    elif q_norm is not None:
         q = q * torch.rsqrt((q * q).mean(-1, keepdim=True) + qk_eps) * q_norm.to(torch.float32)
         k = k * torch.rsqrt((k * k).mean(-1, keepdim=True) + qk_eps) * k_norm.to(torch.float32)
+    if row_scales is not None:
+        q = q * row_scales[:, 0].view(n, 1, 1)
+        k = k * row_scales[:, 1].view(n, 1, 1)
     if rotation is not None:
         c, s = rotation.cos[pos][:, None, :], rotation.sin[pos][:, None, :]
         q = _turn(q, c, s, rotation.rotary_dim, rotation.interleaved)
@@ -325,7 +366,7 @@ def qkv_prepare(qkv, n_heads, n_kv, head_dim, value_dim, positions, act_dtype, q
 
 
 def attention_masked(q, n_heads, n_kv, head_dim, value_dim, k_cache, v_cache, page_size, scale, ctx, group, window=0,
-                     keep_first=0, softcap=0.0, value_rotation=None, gate=None, gate_col=0, gate_elems=1, distance_bias=None):
+                     keep_first=0, softcap=0.0, value_rotation=None, gate=None, gate_col=0, gate_elems=1, distance_bias=None, sink=None):
     n = q.shape[0]
     positions, token_seq = ctx.arrays["positions"], ctx.arrays["token_seq"]
     bt = ctx.arrays[f"block_table_g{group}"]
@@ -348,7 +389,11 @@ def attention_masked(q, n_heads, n_kv, head_dim, value_dim, k_cache, v_cache, pa
                 s = softcap * torch.tanh(s / softcap)
             if distance_bias is not None:
                 s = s + distance_bias[(pos - j).clamp(max=distance_bias.shape[0] - 1).long(), h]
-            out[t, h] = torch.softmax(s, dim=0) @ v[:, g, :]
+            if sink is not None:  # one more term in the denominator, with no value
+                w = torch.softmax(torch.cat([s, sink[h].to(torch.float32).view(1)]), dim=0)[:-1]
+            else:
+                w = torch.softmax(s, dim=0)
+            out[t, h] = w @ v[:, g, :]
     out = attention_finish(out, positions, n_heads, value_dim, value_rotation, gate, gate_col, gate_elems)
     return out.reshape(n, n_heads * value_dim).to(q.dtype)
 
@@ -412,20 +457,40 @@ def rglru(u, y, x, wa_t, ba, wi_t, bi, lam, rate, s_state, conv_state, taps, ctx
     return out.to(u.dtype)
 
 
-def moe_experts(x, token_ids, table, w_gate_up, w_down, activation):
-    """``token_ids`` None: ``table`` has a row per token and ``x`` a row per (token, choice)."""
+def plain_kind(activation):
+    return {"silu": 0, "gelu_tanh": 1, "relu2": 2}[activation]
+
+
+def plain_act(u, activation):
+    if activation == "relu2":
+        r = torch.relu(u)
+        return r * r
+    if activation == "silu":
+        return u * torch.sigmoid(u)
+    k = math.sqrt(2.0 / math.pi)
+    return 0.5 * u * (1.0 + torch.tanh(k * (u + 0.044715 * u * u * u)))
+
+
+def moe_experts(x, token_ids, table, w_gate_up, w_down, activation, input_per_token=False):
+    """``token_ids`` None: ``table`` has a row per token and ``x`` a row per (token, choice), or, with
+    ``input_per_token``, a row per token.  ``w_gate_up`` [experts, 1, ff, hidden]: experts without a gate,
+    down(act(up x)) with a plain activation."""
     top = table.shape[1]
     hidden = x.shape[1]
     n = x.shape[0] if token_ids is not None else table.shape[0]
     rows = torch.empty((n * top, hidden), dtype=torch.float32, device=x.device)
     xf = x.to(torch.float32)
+    gated = w_gate_up.shape[1] == 2
     for t in range(n):
         for k in range(top):
             e = int(table[int(token_ids[t]) if token_ids is not None else t, k])
-            xin = xf[t] if token_ids is not None else xf[t * top + k]
-            g = w_gate_up[e, 0].to(torch.float32) @ xin
-            u = w_gate_up[e, 1].to(torch.float32) @ xin
-            yv = gated_pair(g, u, activation).to(x.dtype).to(torch.float32)
+            xin = xf[t] if (token_ids is not None or input_per_token) else xf[t * top + k]
+            if gated:
+                g = w_gate_up[e, 0].to(torch.float32) @ xin
+                u = w_gate_up[e, 1].to(torch.float32) @ xin
+                yv = gated_pair(g, u, activation).to(x.dtype).to(torch.float32)
+            else:
+                yv = plain_act(w_gate_up[e, 0].to(torch.float32) @ xin, activation).to(x.dtype).to(torch.float32)
             rows[t * top + k] = w_down[e].to(torch.float32) @ yv
     return rows
 
@@ -441,6 +506,8 @@ RefOps.attention_finish = staticmethod(attention_finish)
 RefOps.causal_conv = staticmethod(causal_conv)
 RefOps.rglru = staticmethod(rglru)
 RefOps.moe_experts = staticmethod(moe_experts)
+RefOps.plain_kind = staticmethod(plain_kind)
+RefOps.qk_row_scales = staticmethod(qk_row_scales)
 
 
 # ------------------------------------------------- norms on both sides of a branch, plain feed-forward
@@ -612,24 +679,33 @@ def gated_head_norm(o, weight, eps, gate, gate_col, n_heads, vdim, out_dtype, ga
     return (y * g * torch.sigmoid(g)).to(out_dtype)
 
 
-def moe_router_topk(logits, x, top, experts=None):
+def moe_router_topk(logits, x, top, experts=None, bias=None, scores="sigmoid"):
+    """``scores`` "sigmoid": (choice, x's rows once per chosen expert times sigmoid(logit)); "softmax_of_chosen":
+    (choice, float32 weights [N, top], the softmax over the chosen logits alone); ``bias`` joins the logits first."""
     experts = logits.shape[1] if experts is None else experts
     z = logits[:, :experts].float()
+    if bias is not None:
+        z = z + bias.float()
     n = z.shape[0]
-    choice = torch.empty((n, top), dtype=torch.int32, device=x.device)
-    xs = torch.empty((n * top, x.shape[1]), dtype=x.dtype, device=x.device)
+    choice = torch.empty((n, top), dtype=torch.int32, device=logits.device)
     for t in range(n):
         left = z[t].clone()
         for k in range(top):
             e = int(torch.argmax(left))  # (the first of equals)
             choice[t, k] = e
-            xs[t * top + k] = (x[t].float() * torch.sigmoid(z[t, e])).to(x.dtype)
             left[e] = -math.inf
+    chosen = torch.gather(z, 1, choice.long())
+    if scores == "softmax_of_chosen":
+        return choice, torch.softmax(chosen, dim=1)
+    xs = (x.float()[:, None, :] * torch.sigmoid(chosen)[:, :, None]).to(x.dtype).reshape(n * top, x.shape[1])
     return choice, xs
 
 
-def moe_combine(dense, rows, top, weight=1.0):
-    out = rows.view(rows.shape[0] // top, top, rows.shape[1]).sum(1) * weight
+def moe_combine(dense, rows, top, weight=1.0, row_weights=None):
+    r = rows.view(rows.shape[0] // top, top, rows.shape[1])
+    if row_weights is not None:
+        r = r * row_weights.view(-1, top, 1)
+    out = r.sum(1) * weight
     return out if dense is None else out + dense.float()
 
 

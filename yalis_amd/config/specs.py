@@ -63,10 +63,13 @@ class RunEntry:
     """One entry of the run order.  ``layer`` indexes ``ModelSpec.layers`` and may
     occur in several entries (shared weights, separate caches).  ``cache_from``
     names an earlier entry whose cache this entry's mixer reads instead of
-    keeping one of its own."""
+    keeping one of its own.  ``added_row`` = (tensor name, row, rows): before the entry
+    runs, row ``row`` of the checkpoint table [rows, hidden] is added to every token's
+    stream (a learned vector per pass over a stretch of layers that runs several times)."""
 
     layer: int
     cache_from: Optional[int] = None
+    added_row: Optional[Tuple[str, int, int]] = None
 
 
 @dataclass(frozen=True)
@@ -93,6 +96,11 @@ class ModelSpec:
                     raise ValueError(
                         f"run_order[{i}].cache_from={e.cache_from} must name an earlier entry"
                     )
+            if e.added_row is not None:
+                name, row, rows = e.added_row
+                if not 0 <= row < rows:
+                    raise ValueError(f"run_order[{i}].added_row names row {row} of the {rows} of {name!r}")
+            if e.cache_from is not None:
                 if self.run_order[e.cache_from].cache_from is not None:
                     raise ValueError(
                         f"run_order[{i}].cache_from={e.cache_from} names an entry that itself borrows a cache"

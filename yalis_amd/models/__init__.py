@@ -1,2 +1,2 @@
 """Architectures.  Importing the package registers the ones it ships."""
-from . import llama, mesolix, nutavik, suranex  # noqa: F401
+from . import bekedra, llama, mesolix, nutavik, suranex  # noqa: F401

@@ -15,7 +15,7 @@ import torch
 from ..config.specs import ModelSpec
 from ..parts import BLOCKS, EMBEDDINGS, HEADS, NORMS
 from ..parts.base import FAMILIES
-from ..parts.base import KVNeed, Runtime, StateNeed
+from ..parts.base import KVNeed, PlusRow, Runtime, StateNeed
 from ..weights.loader import TensorSpec
 
 
@@ -78,6 +78,14 @@ class DecoderModel:
                 built[role] = FAMILIES[family].get(part.kind)(params, rt)
             self.blocks.append(arrangement(**built, **dict(ls.params)))
 
+        # tables of which a run entry adds one row to the stream before it runs: name -> rows
+        self.added_tables: Dict[str, int] = {}
+        for e in spec.run_order:
+            if e.added_row is not None:
+                name, _, rows = e.added_row
+                if self.added_tables.setdefault(name, rows) != rows:
+                    raise ValueError(f"run entries name the table {name!r} with different numbers of rows")
+        self._added: Dict[str, torch.Tensor] = {}
         self.cache_groups, self.state_needs, self.sites = self._plan_memory()
         # a step may be replayed from a captured graph only if every part allows it
         self.graph_capturable = all(getattr(p, "graph_capturable", False) for p in self.all_parts())
@@ -134,7 +142,8 @@ class DecoderModel:
         yield self.head
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
-        out: Dict[str, TensorSpec] = {}
+        out: Dict[str, TensorSpec] = {name: TensorSpec((rows, self.spec.hidden_size), "float", ("normal", 0.5))
+                                      for name, rows in self.added_tables.items()}
         for p in self.all_parts():
             for name, spec in p.tensor_specs().items():
                 if name in out and out[name].shape != spec.shape:
@@ -144,7 +153,7 @@ class DecoderModel:
 
     def tensor_uses(self) -> Dict[str, int]:
         """How many parts ask for each tensor (a tied table is asked for twice)."""
-        out: Dict[str, int] = {}
+        out: Dict[str, int] = {name: 1 for name in self.added_tables}
         for p in self.all_parts():
             for name in p.tensor_specs():
                 out[name] = out.get(name, 0) + 1
@@ -153,6 +162,8 @@ class DecoderModel:
     def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
         """Every part takes its tensors from ``tensors``: a dict, or a source that makes
         each tensor when it is asked for (each part asks once for each of its names)."""
+        for name in self.added_tables:
+            self._added[name] = tensors[name].contiguous()
         for p in self.all_parts():
             p.load(tensors)
 
@@ -171,10 +182,13 @@ class DecoderModel:
         if getattr(self.embedding, "needs_positions", False):
             residual, delta = self.embedding.forward(ctx.arrays["token_ids"], ctx.arrays["positions"]), None
         elif begin is not None:
-            residual, delta = begin(ctx.arrays["token_ids"], bool(getattr(first, "takes_embedded_rows", False)))
+            lazily = bool(getattr(first, "takes_embedded_rows", False)) and self.spec.run_order[0].added_row is None
+            residual, delta = begin(ctx.arrays["token_ids"], lazily)
         else:
             residual, delta = self.embedding.forward(ctx.arrays["token_ids"]), None
         for i, e in enumerate(self.spec.run_order):
+            if e.added_row is not None:  # the block's first norm adds the row with whatever is pending
+                delta = PlusRow(delta, self._added[e.added_row[0]][e.added_row[1]])
             delta = self.blocks[e.layer].forward(residual, delta, ctx, ctx.site(i))
         rows = ctx.arrays["logit_rows"]
         if rows.numel() == 0:

@@ -30,7 +30,16 @@ prefix, [buckets, num_heads]; "far": D; "buckets": B or None, the tensor's rows}
 head added to the scaled score of a key n positions back, row bucket(n) of the tensor with bucket(n) =
 n below B/2 and min(B - 1, B/2 + floor(ln(n / (B/2)) / ln(D / (B/2)) * (B - B/2))) from there on, so
 that distances up to B/2 have a row each and the rows beyond cover distances that grow
-geometrically up to D).  A layer may have no position encoding at all (``position`` None).
+geometrically up to D), sink (a tensor name below the prefix, [num_heads]: exp(sink_h) joins the
+softmax's denominator of head h once; it has no key and no value and is neither scaled nor squashed),
+values_from_keys (True: there is no v projection; a token's values are its keys as projected, with
+their bias and before any norm; value_dim = head_dim), projection_bias ({"q": name, "k": name}:
+biases of the q and k projections below the prefix, added in float32 before everything else),
+qk_norm["over"] ("head", the default, or "projection": one RMS norm over all of a token's query
+heads together, and one over all its key heads, with weights as wide as the projections),
+query_temperature ({"coef": c, "every": e}: the query at position p is multiplied by
+1 + c ln(floor((p + 1) / e) + 1), after the norm).  A layer may have no position encoding at all
+(``position`` None).
 """
 from __future__ import annotations
 
@@ -92,14 +101,31 @@ class Attention(Mixer):
         self.gate_elems = self.value_dim if self.gate_per == "element" else 1
         self.distance_bias = params.get("distance_bias")
         self.bias_by_distance = None
+        self.sink_name = params.get("sink")
+        self.sink = None
+        self.values_from_keys = bool(params.get("values_from_keys", False))
+        if self.values_from_keys and self.value_dim != self.head_dim:
+            raise ValueError(f"{self.prefix}: values that are the keys are as wide as the keys")
+        self.projection_bias = dict(params.get("projection_bias") or {})
+        if set(self.projection_bias) - {"q", "k"}:
+            raise ValueError(f"{self.prefix}: projection_bias names the biases of q and k")
+        self.norm_over_projection = bool(self.qk_norm) and self.qk_norm.get("over", "head") == "projection"
+        if self.qk_norm and self.qk_norm.get("over", "head") not in ("head", "projection"):
+            raise ValueError(f"{self.prefix}: qk_norm is over 'head' or 'projection'")
+        self.query_temperature = params.get("query_temperature")
+        if self.query_temperature is not None and int(self.query_temperature["every"]) < 1:
+            raise ValueError(f"{self.prefix}: query_temperature every must be at least 1")
+        self.b_proj = None
         self.masked = bool(
             self.value_dim != self.head_dim or self.qk_norm or self.value_norm_eps is not None or self.value_rotation is not None
-            or self.softcap or self.keep_first or self.gate_name or self.distance_bias
+            or self.softcap or self.keep_first or self.gate_name or self.distance_bias or self.sink_name or self.values_from_keys
+            or self.projection_bias or self.query_temperature
         )
         self.w_qn = self.w_kn = None
         if self.masked:
             if self.bias:
-                raise ValueError(f"{self.prefix}: biases are not offered together with the masked attention's options")
+                raise ValueError(f"{self.prefix}: the four biases are not offered together with the masked attention's options "
+                                 "(projection_bias gives q and k theirs)")
             self.group = None
             self.w_qkv = self.w_q = self.w_o = None
             self.b_qkv = self.b_q = self.b_o = None
@@ -108,6 +134,9 @@ class Attention(Mixer):
             # values of 64 or 128 elements alike); everything else runs on the general float32-arithmetic kernel
             can = getattr(rt.ops, "attention_can_rotate", None)
             self.on_matrix_cores = bool(can is not None and self.value_dim == self.head_dim and can(rt.act_dtype, self.head_dim) is True)
+            if self.on_matrix_cores and self.sink_name:
+                with_sink = getattr(rt.ops, "attention_takes_sink", None)
+                self.on_matrix_cores = bool(with_sink is not None and with_sink(rt.act_dtype, self.head_dim) is True)
             if self.on_matrix_cores:
                 self._tile_sizes(rt)
             return
@@ -142,11 +171,19 @@ class Attention(Mixer):
         }
         if self.projects_kv:
             specs[self.names["k"]] = TensorSpec((kd, self.hidden))
-            specs[self.names["v"]] = TensorSpec((self.n_kv * self.value_dim, self.hidden))
+            if not self.values_from_keys:
+                specs[self.names["v"]] = TensorSpec((self.n_kv * self.value_dim, self.hidden))
         if self.qk_norm:
-            specs[f"{self.prefix}.{self.qk_norm['q']}"] = TensorSpec((self.head_dim,), "float", ("one_plus_normal", 0.1))
+            qn, kn = (hd, kd) if self.norm_over_projection else (self.head_dim, self.head_dim)
+            specs[f"{self.prefix}.{self.qk_norm['q']}"] = TensorSpec((qn,), "float", ("one_plus_normal", 0.1))
             if self.projects_kv:
-                specs[f"{self.prefix}.{self.qk_norm['k']}"] = TensorSpec((self.head_dim,), "float", ("one_plus_normal", 0.1))
+                specs[f"{self.prefix}.{self.qk_norm['k']}"] = TensorSpec((kn,), "float", ("one_plus_normal", 0.1))
+        if "q" in self.projection_bias:
+            specs[f"{self.prefix}.{self.projection_bias['q']}"] = TensorSpec((hd,), "float", ("normal", 0.1))
+        if "k" in self.projection_bias and self.projects_kv:
+            specs[f"{self.prefix}.{self.projection_bias['k']}"] = TensorSpec((kd,), "float", ("normal", 0.1))
+        if self.sink_name:
+            specs[f"{self.prefix}.{self.sink_name}"] = TensorSpec((self.n_heads,), "float", ("normal", 1.0))
         if self.gate_name:
             specs[f"{self.prefix}.{self.gate_name}"] = TensorSpec((self.n_heads * self.gate_elems, self.hidden))
         if self.distance_bias:
@@ -169,7 +206,9 @@ class Attention(Mixer):
             # padded to a multiple of 8 so that the few-row product's tiles take it
             parts = [q]
             if self.projects_kv:
-                parts += [tensors[self.names["k"]], tensors[self.names["v"]]]
+                parts.append(tensors[self.names["k"]])
+                if not self.values_from_keys:
+                    parts.append(tensors[self.names["v"]])
             if self.gate_name:
                 parts.append(tensors[f"{self.prefix}.{self.gate_name}"])
             rows = sum(p.shape[0] for p in parts)
@@ -183,6 +222,17 @@ class Attention(Mixer):
                 self.w_kn = tensors[f"{self.prefix}.{self.qk_norm['k']}"] if self.projects_kv else self.w_qn
             if self.distance_bias:
                 self.bias_by_distance = self._bias_by_distance(tensors[f"{self.prefix}.{self.distance_bias['name']}"])
+            if self.sink_name:
+                self.sink = tensors[f"{self.prefix}.{self.sink_name}"].to(torch.float32).contiguous()
+            if self.projection_bias:
+                # one float32 vector over the projection's columns: the biases where they are, zeros elsewhere
+                b = torch.zeros(self.w_qkv.shape[0], dtype=torch.float32, device=q.device)
+                if "q" in self.projection_bias:
+                    b[: q.shape[0]] = tensors[f"{self.prefix}.{self.projection_bias['q']}"].to(torch.float32)
+                if "k" in self.projection_bias and self.projects_kv:
+                    kd = self.n_kv * self.head_dim
+                    b[q.shape[0]: q.shape[0] + kd] = tensors[f"{self.prefix}.{self.projection_bias['k']}"].to(torch.float32)
+                self.b_proj = b
             return
         if self.projects_kv:
             self.w_qkv = torch.cat([q, tensors[self.names["k"]], tensors[self.names["v"]]], dim=0).contiguous()
@@ -228,7 +278,8 @@ class Attention(Mixer):
     def products(self):
         hd, kd = self.n_heads * self.head_dim, self.n_kv * self.head_dim
         if self.masked:
-            rows = hd + (kd + self.n_kv * self.value_dim if self.projects_kv else 0) + (self.n_heads * self.gate_elems if self.gate_name else 0)
+            v_rows = 0 if self.values_from_keys else self.n_kv * self.value_dim
+            rows = hd + (kd + v_rows if self.projects_kv else 0) + (self.n_heads * self.gate_elems if self.gate_name else 0)
             return ((rows + (-rows % 16), self.hidden), (self.hidden, self.n_heads * self.value_dim))
         return ((hd + 2 * kd if self.projects_kv else hd, self.hidden), (self.hidden, hd))
 
@@ -273,14 +324,30 @@ class Attention(Mixer):
         proj = ops.linear(h, self.w_qkv, self.rt.act_dtype, partial_ok=True)
         n_kv_rows = self.n_kv if site.owns_cache else 0
         k_cache, v_cache = site.kv()
+        more = {}
+        if self.norm_over_projection or self.query_temperature is not None:
+            # what a token's queries and keys are multiplied with as wholes: the inverse root mean square over all
+            # heads at once, and the temperature of the token's position
+            temp = self.query_temperature
+            more["row_scales"] = ops.qk_row_scales(
+                proj, self.n_heads * self.head_dim, n_kv_rows * self.head_dim, ctx.arrays["positions"], bias=self.b_proj,
+                eps=float(self.qk_norm["eps"]) if self.norm_over_projection else None,
+                temperature=None if temp is None else (float(temp["coef"]), int(temp["every"])))
+        if self.norm_over_projection:
+            more["norm_over_projection"] = True
+        if self.b_proj is not None:
+            more["bias"] = self.b_proj
+        if self.values_from_keys:
+            more["values_from_keys"] = True
         q = ops.qkv_prepare(
             proj, self.n_heads, n_kv_rows, self.head_dim, self.value_dim, ctx.arrays["positions"], self.rt.act_dtype,
             q_norm=self.w_qn, k_norm=self.w_kn, qk_eps=float(self.qk_norm["eps"]) if self.qk_norm else 0.0,
             rotation=self.rotation, value_norm_eps=self.value_norm_eps, value_rotation=self.value_rotation,
             k_cache=k_cache, v_cache=v_cache, slots=ctx.arrays[f"slots_g{site.group}"] if n_kv_rows else None,
-            page_size=self.rt.page_size,
+            page_size=self.rt.page_size, **more,
         )
-        gate_col = self.n_heads * self.head_dim + n_kv_rows * (self.head_dim + self.value_dim)
+        gate_col = self.n_heads * self.head_dim + n_kv_rows * (self.head_dim + (0 if self.values_from_keys else self.value_dim))
+        sink = {} if self.sink is None else {"sink": self.sink}
         if self.on_matrix_cores:
             memo_key = f"attention_long_col_tiles_{self.layout}"
             col_tiles = ctx.memo.get(memo_key)
@@ -292,7 +359,7 @@ class Attention(Mixer):
                 ctx.arrays[f"attention_tiles_{self.tokens_per_tile}_upto{self.long_tile}"],
                 ctx.arrays[f"attention_long_tiles_{self.long_tile_2 if col_tiles == 2 else self.long_tile}_{self.layout}"],
                 long_col_tiles=col_tiles, keep_first=self.keep_first if self.window else 0, softcap=self.softcap,
-                distance_bias=self.bias_by_distance,
+                distance_bias=self.bias_by_distance, **sink,
             )
             if self.value_rotation is not None or self.gate_name:
                 ops.attention_finish(out, ctx.arrays["positions"], self.n_heads, self.value_dim, self.value_rotation,
@@ -302,7 +369,7 @@ class Attention(Mixer):
             q, self.n_heads, self.n_kv, self.head_dim, self.value_dim, k_cache, v_cache, self.rt.page_size, self.scale, ctx,
             site.group, window=0 if self.window is None else int(self.window), keep_first=self.keep_first,
             softcap=self.softcap, value_rotation=self.value_rotation, gate=proj if self.gate_name else None, gate_col=gate_col,
-            gate_elems=self.gate_elems, distance_bias=self.bias_by_distance,
+            gate_elems=self.gate_elems, distance_bias=self.bias_by_distance, **sink,
         )
         return ops.linear(out, self.w_o, self.rt.act_dtype, partial_ok=True)
 

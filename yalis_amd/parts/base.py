@@ -100,6 +100,25 @@ class NormedBranch:
         self.norm.norm_add(residual, self.branch, scale=self.scale)
 
 
+class PlusRow:
+    """A pending contribution (``inner``: whatever a block handed on, or None) together with one
+    vector ``row`` [hidden] that every token's stream receives as well: ``residual += inner + row``.
+    A norm that understands it adds both in the pass that norms the stream; ``settle`` adds them for
+    whoever cannot and returns what is then left to add (nothing)."""
+
+    def __init__(self, inner, row: torch.Tensor):
+        self.inner, self.row = inner, row
+
+    def settle(self, residual: torch.Tensor):
+        inner = self.inner
+        if isinstance(inner, NormedBranch):
+            inner = inner.settle(residual)
+        if inner is not None and not isinstance(inner, Settled):
+            residual += inner.float()
+        residual += self.row.to(torch.float32)
+        return None
+
+
 class Part:
     """Common to all parts."""
 
@@ -161,15 +180,20 @@ class FeedForward(Part):
 class ExpertRows:
     """A feed-forward's output not yet summed: ``dense`` (a tensor, a product's unreduced slices,
     or None) plus ``weight`` times the sum of each token's ``top`` consecutive rows of ``rows``
-    (float32 [tokens * top, width]).  A norm's ``norm_add`` sums them while it reads them;
-    ``combine()`` gives the tensor for whoever cannot."""
+    (float32 [tokens * top, width]), each row first multiplied by its own entry of ``row_weights``
+    (float32 [tokens, top]) where those are given.  A norm's ``norm_add`` sums them while it reads
+    them; ``combine()`` gives the tensor for whoever cannot."""
 
-    def __init__(self, dense, rows: torch.Tensor, top: int, weight: float):
+    def __init__(self, dense, rows: torch.Tensor, top: int, weight: float, row_weights: Optional[torch.Tensor] = None):
         self.dense, self.rows, self.top, self.weight = dense, rows, int(top), float(weight)
+        self.row_weights = row_weights
         self.shape = (rows.shape[0] // self.top, rows.shape[1])
 
     def combine(self) -> torch.Tensor:
-        out = self.rows.view(self.shape[0], self.top, self.shape[1]).sum(1) * self.weight
+        rows = self.rows.view(self.shape[0], self.top, self.shape[1])
+        if self.row_weights is not None:
+            rows = rows * self.row_weights.view(self.shape[0], self.top, 1)
+        out = rows.sum(1) * self.weight
         if self.dense is not None:
             out = out + self.dense.float()
         return out

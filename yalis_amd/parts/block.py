@@ -12,7 +12,7 @@ returns its own last contribution, to be added by whoever comes next.
 """
 from __future__ import annotations
 
-from .base import Block, NormedBranch, Settled, register_block
+from .base import Block, ExpertRows, NormedBranch, PlusRow, Settled, register_block
 
 
 @register_block("prenorm")
@@ -45,6 +45,42 @@ class PreNormBlock(Block):
         return self.feed_forward.forward(h, ctx)
 
 
+@register_block("parallel")
+class ParallelBlock(Block):
+    """One norm that both branches read: h = norm(x); x = x + (mixer(h) + feed_forward(h)).  A layer may leave
+    the feed-forward out.  The two outputs are summed in float32 by one kernel (``ops.moe_combine``: the mixer's
+    output, possibly still a product's unreduced slices, plus a mixture's uncombined rows times their weights) and
+    handed on as one pending contribution."""
+
+    roles = {
+        "norm": ("norm", True),
+        "mixer": ("mixer", True),
+        "feed_forward": ("feed_forward", False),
+    }
+
+    def __init__(self, norm, mixer, feed_forward=None):
+        self.norm = norm
+        self.mixer = mixer
+        self.feed_forward = feed_forward
+
+    @property
+    def takes_embedded_rows(self):
+        return bool(getattr(self.norm, "takes_embedded_rows", False))
+
+    def forward(self, residual, delta, ctx, site):
+        h = self.norm.add_norm(residual, delta)
+        a = self.mixer.forward(h, ctx, site)
+        if self.feed_forward is None:
+            return a
+        f = self.feed_forward.forward(h, ctx)
+        ops = self.mixer.rt.ops
+        if not isinstance(f, ExpertRows):  # any other feed-forward: its output is one row a token
+            f = ExpertRows(None, f.float().contiguous(), 1, 1.0)
+        if f.dense is not None:
+            a = ops.moe_combine(a, f.dense.float().contiguous(), 1, 1.0)
+        return ops.moe_combine(a, f.rows, f.top, f.weight, row_weights=f.row_weights)
+
+
 @register_block("branch_norm")
 class BranchNormBlock(Block):
     """Norms on the branches' outputs only: x = x + norm_1(mixer(x)); x = x + norm_2(feed_forward(x)).
@@ -71,6 +107,8 @@ class BranchNormBlock(Block):
         self.feed_forward_norm = feed_forward_norm
 
     def forward(self, residual, delta, ctx, site):
+        if isinstance(delta, PlusRow):
+            delta = delta.settle(residual)
         if isinstance(delta, Settled):
             h = delta.activations
         else:

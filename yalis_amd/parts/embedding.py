@@ -18,7 +18,7 @@ from .base import Part, Runtime, register_embedding, register_head
 
 @register_embedding("token_embedding")
 class TokenEmbedding(Part):
-    """params: name, vocab_size, hidden_size."""
+    """params: name, vocab_size, hidden_size, scale (1.0: what a token's row is multiplied with, in float32)."""
 
     graph_capturable = True
 
@@ -27,6 +27,7 @@ class TokenEmbedding(Part):
         self.name = params["name"]
         self.vocab = int(params["vocab_size"])
         self.hidden = int(params["hidden_size"])
+        self.scale = float(params.get("scale", 1.0))
         self.table = None
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
@@ -37,6 +38,8 @@ class TokenEmbedding(Part):
 
     def forward(self, token_ids: torch.Tensor) -> torch.Tensor:
         """The float32 residual stream [N, hidden]."""
+        if self.scale != 1.0:
+            return self.rt.ops.embed(token_ids, self.table, scale=self.scale)
         return self.rt.ops.embed(token_ids, self.table)
 
     def begin(self, token_ids: torch.Tensor, lazily: bool):
@@ -45,7 +48,7 @@ class TokenEmbedding(Part):
         rows as a pending contribution that the first norm's kernel gathers itself (a block says
         through ``takes_embedded_rows`` whether its first norm does)."""
         make = getattr(self.rt.ops, "embedded_rows", None)
-        if lazily and make is not None:
+        if lazily and make is not None and self.scale == 1.0:
             return make(token_ids, self.table)
         return self.forward(token_ids), None
 

@@ -115,9 +115,17 @@ class RoutedMoE(FeedForward):
     ``ops.moe_experts`` with the router's choice as their table; one kernel sums a token's rows and the shared
     expert's output (``ops.moe_combine``).
 
+    Other forms of the same mixture: ``router_bias`` (a tensor name below the prefix, [experts], added to the
+    float32 logits before the choice), ``scores`` "softmax_of_chosen" (the chosen experts' weights are the softmax
+    over their own logits alone; the default "sigmoid" is as above), ``weighs`` "output" (an expert reads the
+    token's input as it is and its output is multiplied by the weight; the default "input" is as above),
+    ``gated`` False (an expert is down(act(up x)) with ``activation`` one of the kernel library's plain ones,
+    "relu2" the square of relu; no gate tensor).  With weights on the outputs ``forward`` returns the experts'
+    uncombined rows beside their weights (``ExpertRows``) for whoever sums the branch into the stream.
+
     params: prefix, hidden_size, experts, top, intermediate_size, activation ("silu"), shared (None or
-    {"intermediate_size", "activation"}), names (optional: "router", "expert" with {e} for the expert's number,
-    "shared", "gate", "up", "down")."""
+    {"intermediate_size", "activation"}), router_bias (None), scores ("sigmoid"), weighs ("input"), gated (True),
+    names (optional: "router", "expert" with {e} for the expert's number, "shared", "gate", "up", "down")."""
 
     graph_capturable = True
 
@@ -131,7 +139,18 @@ class RoutedMoE(FeedForward):
         self.activation = params.get("activation", "silu")
         if not 1 <= self.top <= self.experts:
             raise ValueError(f"{self.prefix}: top={self.top} of {self.experts} experts")
-        rt.ops.gated_kind(self.activation)
+        self.gated = bool(params.get("gated", True))
+        if self.gated:
+            rt.ops.gated_kind(self.activation)
+        else:
+            rt.ops.plain_kind(self.activation)  # raises for one the kernels do not know
+        self.router_bias_name = params.get("router_bias")
+        self.router_bias = None
+        self.scores = params.get("scores", "sigmoid")
+        self.weighs = params.get("weighs", "input")
+        if (self.scores, self.weighs) not in (("sigmoid", "input"), ("softmax_of_chosen", "output")):
+            raise ValueError(f"{self.prefix}: scores={self.scores!r} with weighs={self.weighs!r} is not offered "
+                             "(sigmoid scores weigh the inputs, a softmax over the chosen weighs the outputs)")
         self.shared = params.get("shared")
         names = {"router": "router", "expert": "e{e}", "shared": "shared", "gate": "gate", "up": "up", "down": "down"}
         names.update(params.get("names", {}))
@@ -150,8 +169,11 @@ class RoutedMoE(FeedForward):
     def tensor_specs(self) -> Dict[str, TensorSpec]:
         # (random routers are made wide enough that tokens differ in what they choose)
         specs = {f"{self.prefix}.{self.names['router']}": TensorSpec((self.experts, self.hidden), "float", ("normal", 0.5))}
+        if self.router_bias_name:
+            specs[f"{self.prefix}.{self.router_bias_name}"] = TensorSpec((self.experts,), "float", ("normal", 0.5))
         for e in range(self.experts):
-            specs[self._name(self._expert(e), "gate")] = TensorSpec((self.inter, self.hidden))
+            if self.gated:
+                specs[self._name(self._expert(e), "gate")] = TensorSpec((self.inter, self.hidden))
             specs[self._name(self._expert(e), "up")] = TensorSpec((self.inter, self.hidden))
             specs[self._name(self._expert(e), "down")] = TensorSpec((self.hidden, self.inter))
         if self.shared:
@@ -167,8 +189,11 @@ class RoutedMoE(FeedForward):
         if pad:
             router = torch.cat([router, torch.zeros((pad, self.hidden), dtype=router.dtype, device=router.device)], dim=0)
         self.w_router = router.contiguous()
+        if self.router_bias_name:
+            self.router_bias = tensors[f"{self.prefix}.{self.router_bias_name}"].to(torch.float32).contiguous()
+        # [experts, 2, ff, hidden] (gate rows, then up rows), or [experts, 1, ff, hidden] without gates
         self.w_gate_up = torch.stack([
-            torch.stack([tensors[self._name(self._expert(e), "gate")], tensors[self._name(self._expert(e), "up")]])
+            torch.stack(([tensors[self._name(self._expert(e), "gate")]] if self.gated else []) + [tensors[self._name(self._expert(e), "up")]])
             for e in range(self.experts)
         ]).contiguous()
         self.w_down = torch.stack([tensors[self._name(self._expert(e), "down")] for e in range(self.experts)]).contiguous()
@@ -187,7 +212,15 @@ class RoutedMoE(FeedForward):
     def forward(self, h: torch.Tensor, ctx):
         ops = self.rt.ops
         logits = ops.linear(h, self.w_router, torch.float32)
-        choice, scaled = ops.moe_router_topk(logits, h, self.top, experts=self.experts)
+        if self.weighs == "output":
+            choice, weights = ops.moe_router_topk(logits, None, self.top, experts=self.experts, bias=self.router_bias, scores=self.scores)
+            rows = ops.moe_experts(h, None, choice, self.w_gate_up, self.w_down, self.activation, input_per_token=True)
+            dense = None
+            if self.shared:
+                a = ops.gate_up_act(h, self.shared_gate_up, self.shared_group, self.shared.get("activation", "silu"), self.rt.act_dtype)
+                dense = ops.linear(a, self.shared_down, self.rt.act_dtype, partial_ok=True)
+            return ExpertRows(dense, rows, self.top, 1.0, row_weights=weights)
+        choice, scaled = ops.moe_router_topk(logits, h, self.top, experts=self.experts, bias=self.router_bias)
         rows = ops.moe_experts(scaled, None, choice, self.w_gate_up, self.w_down, self.activation)
         dense = None
         if self.shared:

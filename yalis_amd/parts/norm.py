@@ -14,7 +14,7 @@ from typing import Dict, Mapping, Optional
 import torch
 
 from ..weights.loader import TensorSpec
-from .base import ExpertRows, Norm, NormedBranch, Runtime, Settled, register_norm
+from .base import ExpertRows, Norm, NormedBranch, PlusRow, Runtime, Settled, register_norm
 
 
 @register_norm("rmsnorm")
@@ -43,10 +43,15 @@ class RMSNorm(Norm):
         return self.rt.ops.rmsnorm(x, self.weight, self.eps, self.unit_offset, self.rt.act_dtype)
 
     def add_norm(self, residual, delta):
+        row = None
+        if isinstance(delta, PlusRow):  # a vector for every token joins the stream in the same pass
+            delta, row = delta.inner, delta.row
         if isinstance(delta, NormedBranch):
             delta = delta.settle(residual)
         if isinstance(delta, Settled):
             delta = None
+        if row is not None:
+            return self.rt.ops.add_rmsnorm(residual, delta, self.weight, self.eps, self.unit_offset, self.rt.act_dtype, row=row)
         return self.rt.ops.add_rmsnorm(
             residual, delta, self.weight, self.eps, self.unit_offset, self.rt.act_dtype
         )
@@ -54,12 +59,16 @@ class RMSNorm(Norm):
     def norm_add(self, residual, branch, expert_rows=None, expert_weight=1.0, scale=1.0):
         if scale != 1.0:
             raise ValueError("this norm adds its branch unscaled")
+        if isinstance(branch, ExpertRows) and branch.row_weights is not None:
+            branch = branch.combine()  # (rows with weights of their own are summed first)
         if isinstance(branch, ExpertRows):
             branch, expert_rows, expert_weight = branch.dense, branch.rows, branch.weight
         return self.rt.ops.norm_add(residual, branch, self.weight, self.eps, self.unit_offset, self.rt.act_dtype,
                                     expert_rows=expert_rows, expert_weight=expert_weight)
 
     def gather_add_norm(self, residual, delta, rows):
+        if isinstance(delta, PlusRow):
+            delta = delta.settle(residual)
         if isinstance(delta, NormedBranch):
             delta = delta.settle(residual)
         if isinstance(delta, Settled):
@@ -111,6 +120,8 @@ class LayerNorm(Norm):
 
     def _pending(self, residual, delta):
         """(branch, its norm's constants or None, scale) of a pending contribution."""
+        if isinstance(delta, PlusRow):
+            delta = delta.settle(residual)
         if isinstance(delta, Settled) or delta is None:
             return None, None, 1.0
         if isinstance(delta, NormedBranch):
