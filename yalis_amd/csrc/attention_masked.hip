@@ -5,7 +5,12 @@
 //    shared by the heads, or none), rotary positions on the first rotary_dim elements of queries
 //    and keys, values divided by their root mean square per head, values rotated by their own
 //    table over all of value_dim; queries go to a tensor, keys and values into the pages.
-//    Every option can be left out; with none of them it is rotary + append.
+//    Every option can be left out; with none of them it is rotary + append.  More options: a float32 bias per
+//    column of the projection, added first; values that are the keys as projected (with the bias, before the norm:
+//    the projection then has no value columns); the norm over all of a token's query heads at once (and over all
+//    its key heads), with weights as wide as the projections, whose inverse root mean square comes from
+//  * yk_qk_row_scales: per token, what its queries and its keys are multiplied with as wholes after the weights:
+//    that inverse root mean square and / or the queries' temperature 1 + coef ln(floor((p + 1) / every) + 1).
 //  * yk_attn_masked: scores q . k * scale, optionally squashed s <- cap * tanh(s / cap); key j
 //    is visible to the query at position p iff j <= p and (p - j < window or j < keep_first)
 //    (window 0: no window); softmax over the visible keys; keys of head_dim, values of
@@ -51,7 +56,8 @@ __global__ __launch_bounds__(256) void qkv_prepare_kernel(
     int qk_norm, float qk_eps, const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rotary_dim,
     int interleaved, int max_pos, int v_norm, float v_eps, const float* __restrict__ v_cos,
     const float* __restrict__ v_sin, int v_interleaved, int v_max_pos, T* __restrict__ k_cache,
-    T* __restrict__ v_cache, const int32_t* __restrict__ slots, int page_size, int tiled) {
+    T* __restrict__ v_cache, const int32_t* __restrict__ slots, int page_size, int tiled,
+    const float* __restrict__ bias, const float* __restrict__ row_scales, int v_from_k) {
   __shared__ float bufs[4][kMaxHead];
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
   float* buf = bufs[wave];
@@ -63,6 +69,7 @@ __global__ __launch_bounds__(256) void qkv_prepare_kernel(
   int col0;
   if (kind == 0) col0 = slot_y * head_dim;
   else if (kind == 1) col0 = n_heads * head_dim + (slot_y - n_heads) * head_dim;
+  else if (v_from_k) col0 = n_heads * head_dim + (slot_y - n_heads - n_kv) * head_dim;  // the key head's own columns
   else col0 = (n_heads + n_kv) * head_dim + (slot_y - n_heads - n_kv) * v_dim;
   const TS* row = src + static_cast<size_t>(n) * src_stride + col0;
   // the position, this lane's cosines and sines and the token's slot are asked for before the row
@@ -104,11 +111,12 @@ __global__ __launch_bounds__(256) void qkv_prepare_kernel(
     if (d < len) {
       for (int s = 0; s < n_splits; ++s) v += to_f32<TS>(row[s * split_stride + d]);
       v = as_output(v, round_sum);
+      if (bias != nullptr) v += bias[col0 + d];
     }
     val[i] = v;
     ss = fmaf(v, v, ss);
   }
-  const bool normed = kind == 2 ? v_norm != 0 : qk_norm != 0;
+  const bool normed = kind == 2 ? v_norm != 0 : qk_norm == 1;
   if (normed) {
     ss = wave_sum(ss);
     const float inv = 1.f / sqrtf(ss / static_cast<float>(len) + (kind == 2 ? v_eps : qk_eps));
@@ -118,6 +126,20 @@ __global__ __launch_bounds__(256) void qkv_prepare_kernel(
       const int d = lane + 64 * i;
       if (d < len) val[i] = val[i] * inv * (w != nullptr ? to_f32<TW>(w[d]) : 1.f);
     }
+  } else if (kind != 2 && qk_norm == 2) {
+    // the norm over the whole projection: weights as wide as the projection; the inverse root mean square over
+    // all heads is part of the row's scale below
+    const TW* w = kind == 0 ? q_norm_w + col0 : k_norm_w + (col0 - n_heads * head_dim);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int d = lane + 64 * i;
+      if (d < len) val[i] *= to_f32<TW>(w[d]);
+    }
+  }
+  if (kind != 2 && row_scales != nullptr) {
+    const float rs = row_scales[2 * static_cast<size_t>(n) + kind];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) val[i] *= rs;
   }
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
@@ -166,7 +188,8 @@ __global__ __launch_bounds__(512) void qkv_prepare8_kernel(
     int qk_norm, float qk_eps, const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rotary_dim,
     int interleaved, int max_pos, int v_norm, float v_eps, const float* __restrict__ v_cos,
     const float* __restrict__ v_sin, int v_interleaved, int v_max_pos, bf16_t* __restrict__ k_cache,
-    bf16_t* __restrict__ v_cache, const int32_t* __restrict__ slots, int page_size, int tiled, int n_tokens) {
+    bf16_t* __restrict__ v_cache, const int32_t* __restrict__ slots, int page_size, int tiled, int n_tokens,
+    const float* __restrict__ bias, const float* __restrict__ row_scales, int v_from_k) {
   __shared__ float bufs[8][kMaxHead];
   __shared__ __attribute__((aligned(16))) bf16_t outs[8][kMaxHead];
   __shared__ int slot_s[8];
@@ -180,6 +203,7 @@ __global__ __launch_bounds__(512) void qkv_prepare8_kernel(
   int col0;
   if (kind == 0) col0 = slot_y * head_dim;
   else if (kind == 1) col0 = n_heads * head_dim + (slot_y - n_heads) * head_dim;
+  else if (v_from_k) col0 = n_heads * head_dim + (slot_y - n_heads - n_kv) * head_dim;  // the key head's own columns
   else col0 = (n_heads + n_kv) * head_dim + (slot_y - n_heads - n_kv) * v_dim;
   const TS* row = src + static_cast<size_t>(n) * src_stride + col0;
   const int pos = positions[n];
@@ -219,11 +243,12 @@ __global__ __launch_bounds__(512) void qkv_prepare8_kernel(
     if (d < len) {
       for (int s = 0; s < n_splits; ++s) v += to_f32<TS>(row[s * split_stride + d]);
       v = as_output(v, round_sum);
+      if (bias != nullptr) v += bias[col0 + d];
     }
     val[i] = v;
     ss = fmaf(v, v, ss);
   }
-  const bool normed = kind == 2 ? v_norm != 0 : qk_norm != 0;
+  const bool normed = kind == 2 ? v_norm != 0 : qk_norm == 1;
   if (normed) {
     ss = wave_sum(ss);
     const float inv = 1.f / sqrtf(ss / static_cast<float>(len) + (kind == 2 ? v_eps : qk_eps));
@@ -233,6 +258,20 @@ __global__ __launch_bounds__(512) void qkv_prepare8_kernel(
       const int d = lane + 64 * i;
       if (d < len) val[i] = val[i] * inv * (w != nullptr ? to_f32<TW>(w[d]) : 1.f);
     }
+  } else if (kind != 2 && qk_norm == 2) {
+    // the norm over the whole projection: weights as wide as the projection; the inverse root mean square over
+    // all heads is part of the row's scale below
+    const TW* w = kind == 0 ? q_norm_w + col0 : k_norm_w + (col0 - n_heads * head_dim);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int d = lane + 64 * i;
+      if (d < len) val[i] *= to_f32<TW>(w[d]);
+    }
+  }
+  if (kind != 2 && row_scales != nullptr) {
+    const float rs = row_scales[2 * static_cast<size_t>(n) + kind];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) val[i] *= rs;
   }
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
@@ -305,8 +344,12 @@ extern "C" int yk_qkv_prepare(const void* src, int src_dtype, int n_splits, int 
                               int qk_norm, float qk_eps, const float* cos_t, const float* sin_t, int rotary_dim,
                               int interleaved, int max_pos, int v_norm, float v_eps, const float* v_cos,
                               const float* v_sin, int v_interleaved, int v_max_pos, void* k_cache, void* v_cache,
-                              const int32_t* slots, int page_size, int tiled, hipStream_t stream) {
+                              const int32_t* slots, int page_size, int tiled, const float* bias, const float* row_scales,
+                              int v_from_k, hipStream_t stream) {
   YK_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_kv >= 0, "qkv_prepare: bad sizes");
+  YK_REQUIRE(qk_norm >= 0 && qk_norm <= 2 && (qk_norm != 2 || (row_scales != nullptr && q_norm_w != nullptr && (n_kv == 0 || k_norm_w != nullptr))),
+             "qkv_prepare: a norm over the whole projection takes its weights and the rows' scales");
+  YK_REQUIRE(!v_from_k || v_dim == head_dim, "qkv_prepare: values that are the keys are as wide as the keys");
   YK_REQUIRE(head_dim > 0 && head_dim <= kMaxHead && v_dim > 0 && v_dim <= kMaxHead, "qkv_prepare: heads of 1 to 256 elements");
   YK_REQUIRE(rotary_dim >= 0 && rotary_dim <= head_dim && rotary_dim % 2 == 0, "qkv_prepare: rotary_dim must be even and at most head_dim");
   YK_REQUIRE(rotary_dim == 0 || (cos_t != nullptr && sin_t != nullptr && max_pos > 0), "qkv_prepare: rotary tables missing");
@@ -328,7 +371,7 @@ extern "C" int yk_qkv_prepare(const void* src, int src_dtype, int n_splits, int 
         n_heads, n_kv, head_dim, v_dim, positions, static_cast<const TW*>(q_norm_w),                           \
         static_cast<const TW*>(k_norm_w), qk_norm, qk_eps, cos_t, sin_t, rotary_dim, interleaved, max_pos,      \
         v_norm, v_eps, v_cos, v_sin, v_interleaved, v_max_pos, static_cast<bf16_t*>(k_cache),                  \
-        static_cast<bf16_t*>(v_cache), slots, page_size, tiled, n_tokens);                                     \
+        static_cast<bf16_t*>(v_cache), slots, page_size, tiled, n_tokens, bias, row_scales, v_from_k);         \
     return yk_check_launch("qkv_prepare (8 tokens)");                                                          \
   }
     YK_CASE8(YK_F32, float, YK_F32, float)
@@ -345,7 +388,7 @@ extern "C" int yk_qkv_prepare(const void* src, int src_dtype, int n_splits, int 
         n_heads, n_kv, head_dim, v_dim, positions, static_cast<const TW*>(q_norm_w),                          \
         static_cast<const TW*>(k_norm_w), qk_norm, qk_eps, cos_t, sin_t, rotary_dim, interleaved, max_pos,     \
         v_norm, v_eps, v_cos, v_sin, v_interleaved, v_max_pos, static_cast<T*>(k_cache), static_cast<T*>(v_cache), \
-        slots, page_size, tiled);                                                                             \
+        slots, page_size, tiled, bias, row_scales, v_from_k);                                                 \
     return yk_check_launch("qkv_prepare");                                                                    \
   }
   YK_CASE(YK_F32, float, YK_F32, float, YK_F32, float)
@@ -355,6 +398,60 @@ extern "C" int yk_qkv_prepare(const void* src, int src_dtype, int n_splits, int 
   YK_CASE(YK_BF16, bf16_t, YK_BF16, bf16_t, YK_BF16, bf16_t)
 #undef YK_CASE
   return yk_fail("qkv_prepare: unsupported dtype combination");
+}
+
+// ------------------------------------------------------------------ what scales a token's rows as wholes
+// out[n][0] for the queries, out[n][1] for the keys: 1 / sqrt(mean(x^2) + eps) over all n_q_cols query columns (all
+// n_k_cols key columns) of the biased projection when `normed`, times, for the queries, the temperature
+// 1 + coef * ln(floor((p + 1) / every) + 1) of the token's position p when every > 0.  A workgroup a token.
+template <typename TS>
+__global__ __launch_bounds__(256) void qk_row_scales_kernel(
+    const TS* __restrict__ src, int n_splits, size_t split_stride, int round_sum, int src_stride, int n_q_cols, int n_k_cols,
+    const float* __restrict__ bias, int normed, float eps, const int32_t* __restrict__ positions, float temp_coef,
+    int temp_every, float* __restrict__ out) {
+  __shared__ float scratch[17];
+  const int n = blockIdx.x;
+  float sq = 1.f, sk = 1.f;
+  if (normed) {
+    const TS* row = src + static_cast<size_t>(n) * src_stride;
+    float ssq = 0.f, ssk = 0.f;
+    for (int c = threadIdx.x; c < n_q_cols + n_k_cols; c += blockDim.x) {
+      float v = 0.f;
+      for (int s = 0; s < n_splits; ++s) v += to_f32<TS>(row[s * split_stride + c]);
+      v = as_output(v, round_sum);
+      if (bias != nullptr) v += bias[c];
+      if (c < n_q_cols) ssq = fmaf(v, v, ssq);
+      else ssk = fmaf(v, v, ssk);
+    }
+    ssq = block_sum(ssq, scratch);
+    ssk = block_sum(ssk, scratch);
+    sq = 1.f / sqrtf(ssq / static_cast<float>(n_q_cols) + eps);
+    if (n_k_cols > 0) sk = 1.f / sqrtf(ssk / static_cast<float>(n_k_cols) + eps);
+  }
+  if (threadIdx.x == 0) {
+    if (temp_every > 0) sq *= 1.f + temp_coef * logf(static_cast<float>((positions[n] + 1) / temp_every + 1));
+    out[2 * static_cast<size_t>(n)] = sq;
+    out[2 * static_cast<size_t>(n) + 1] = sk;
+  }
+}
+
+extern "C" int yk_qk_row_scales(const void* src, int src_dtype, int n_splits, int round_sum, int src_stride, int n_tokens,
+                                int n_q_cols, int n_k_cols, const float* bias, int normed, float eps, const int32_t* positions,
+                                float temp_coef, int temp_every, float* out, hipStream_t stream) {
+  YK_REQUIRE(n_tokens >= 0 && n_q_cols > 0 && n_k_cols >= 0 && src_stride >= n_q_cols + n_k_cols, "qk_row_scales: bad sizes");
+  YK_REQUIRE(n_splits >= 1 && (n_splits == 1 || src_dtype == YK_F32), "qk_row_scales: unreduced slices must be float32");
+  YK_REQUIRE(temp_every >= 0 && (temp_every == 0 || positions != nullptr) && eps >= 0.f, "qk_row_scales: bad constants");
+  if (n_tokens == 0) return 0;
+  const size_t stride = static_cast<size_t>(n_tokens) * src_stride;
+  if (src_dtype == YK_F32)
+    qk_row_scales_kernel<float><<<n_tokens, 256, 0, stream>>>(static_cast<const float*>(src), n_splits, stride, round_sum, src_stride,
+                                                              n_q_cols, n_k_cols, bias, normed, eps, positions, temp_coef, temp_every, out);
+  else if (src_dtype == YK_BF16)
+    qk_row_scales_kernel<bf16_t><<<n_tokens, 256, 0, stream>>>(static_cast<const bf16_t*>(src), n_splits, stride, round_sum, src_stride,
+                                                               n_q_cols, n_k_cols, bias, normed, eps, positions, temp_coef, temp_every, out);
+  else
+    return yk_fail("qk_row_scales: unsupported dtype");
+  return yk_check_launch("qk_row_scales");
 }
 
 // ------------------------------------------------------------------------------ the finish
@@ -376,7 +473,7 @@ __global__ __launch_bounds__(64) void attn_masked_kernel(
     int n_kv, float scale, float softcap, int window, int keep_first, int tiled, const float* __restrict__ v_cos,
     const float* __restrict__ v_sin, int v_interleaved, int v_max_pos, const TG* __restrict__ gate_src,
     int gate_splits, size_t gate_split_stride, int gate_round, int gate_stride, int gate_col0, int gate_elems,
-    const float* __restrict__ dist_bias, int bias_rows) {
+    const float* __restrict__ dist_bias, int bias_rows, const float* __restrict__ sink) {
   const size_t slab_k = static_cast<size_t>(page_size) * head_dim, slab_v = static_cast<size_t>(page_size) * v_dim;
   __shared__ float qs[kMaxHead];
   __shared__ float os[kMaxHead];
@@ -393,7 +490,8 @@ __global__ __launch_bounds__(64) void attn_masked_kernel(
   for (int d = lane; d < head_dim; d += 64) qs[d] = to_f32<T>(qrow[d]);
   __syncthreads();
   const int32_t* bt = block_table + static_cast<size_t>(seq) * table_width;
-  float m = -INFINITY, l = 0.f;
+  // a sink starts the running maximum and counts once in the sum: exp(sink) in the denominator, with no value
+  float m = sink != nullptr ? sink[h] : -INFINITY, l = sink != nullptr ? 1.f : 0.f;
   float acc[4] = {0.f, 0.f, 0.f, 0.f};
   for (int t0 = 0; t0 < total; t0 += 64) {
     const int idx = t0 + lane;
@@ -468,14 +566,14 @@ __global__ __launch_bounds__(64) void attn_masked_kernel(
 
 // gate_elems: 1, a gate per head in column gate_col0 + h, or v_dim, one per output element in column gate_col0 + h *
 // v_dim + d.  dist_bias [bias_rows][n_heads] float32 or null: what is added to the score of a key at distance n (the
-// last row for every larger distance).
+// last row for every larger distance).  sink [n_heads] float32 or null: exp(sink[h]) joins head h's denominator once.
 extern "C" int yk_attn_masked(const void* q, int q_stride, void* out, const void* k_cache, const void* v_cache, int dtype,
                               const int32_t* positions, const int32_t* token_seq, const int32_t* block_table,
                               int table_width, int n_tokens, int page_size, int head_dim, int v_dim, int n_heads, int n_kv,
                               float scale, float softcap, int window, int keep_first, int tiled, const float* v_cos,
                               const float* v_sin, int v_interleaved, int v_max_pos, const void* gate_src, int gate_dtype,
                               int gate_splits, int gate_round, int gate_stride, int gate_col0, int gate_elems,
-                              const float* dist_bias, int bias_rows, hipStream_t stream) {
+                              const float* dist_bias, int bias_rows, const float* sink, hipStream_t stream) {
   YK_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0, "attn_masked: bad head counts");
   YK_REQUIRE(gate_src == nullptr || gate_elems == 1 || gate_elems == v_dim, "attn_masked: a gate per head or per output element");
   YK_REQUIRE(dist_bias == nullptr || bias_rows >= 1, "attn_masked: an empty table of biases");
@@ -496,7 +594,7 @@ extern "C" int yk_attn_masked(const void* q, int q_stride, void* out, const void
         static_cast<const T*>(v_cache), positions, token_seq, block_table, table_width, page_size, head_dim,   \
         v_dim, n_heads, n_kv, scale, softcap, window, keep_first, tiled, v_cos, v_sin, v_interleaved, v_max_pos, \
         static_cast<const TG*>(gate_src), gate_splits, gstride, gate_round, gate_stride, gate_col0, gate_elems, \
-        dist_bias, bias_rows);                                                                                 \
+        dist_bias, bias_rows, sink);                                                                           \
     return yk_check_launch("attn_masked");                                                                     \
   }
   YK_CASE(YK_F32, float, YK_F32, float)

@@ -138,6 +138,15 @@ __device__ __forceinline__ float act_gelu_tanh(float z) {
   return 0.5f * z * (1.f + tanhf(k * (z + 0.044715f * z * z * z)));
 }
 __device__ __forceinline__ float act_apply(float z, int act) { return act == 0 ? act_silu(z) : act_gelu_tanh(z); }
+// Plain activations: 0 = silu, 1 = gelu (tanh form), 2 = the square of relu.
+#define YK_PLAIN_KINDS 3
+__device__ __forceinline__ float act_plain(float z, int kind) {
+  if (kind == 2) {
+    const float r = fmaxf(z, 0.f);
+    return r * r;
+  }
+  return act_apply(z, kind);
+}
 // A gated pair: what a feed-forward makes of a gate value g and an up value u.  Kinds 0 and 1:
 // act(g) * u.  Kind 2, the clamped swish gate: g' = min(g, p0), u' = clamp(u, -p0, p0),
 // g' * sigmoid(p1 * g') * (u' + 1) (p0 the limit, p1 the slope of the sigmoid).

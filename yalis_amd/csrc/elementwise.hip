@@ -19,7 +19,7 @@ extern "C" int yk_cache_tiled(int dtype, int head_dim, int page_size) { return c
 template <typename T>
 __global__ void embed_kernel(const int32_t* __restrict__ ids, const T* __restrict__ table,
                              float* __restrict__ out, int width, int vocab, const int32_t* __restrict__ positions,
-                             const T* __restrict__ pos_table, int pos_rows) {
+                             const T* __restrict__ pos_table, int pos_rows, float scale) {
   const int n = blockIdx.x;
   int id = ids[n];
   // ids are checked on the host; clamp so that a bad id cannot read out of bounds
@@ -30,10 +30,10 @@ __global__ void embed_kernel(const int32_t* __restrict__ ids, const T* __restric
     int p = positions[n];
     p = p < 0 ? 0 : (p >= pos_rows ? pos_rows - 1 : p);
     const T* ps = pos_table + static_cast<size_t>(p) * width;
-    for (int c = threadIdx.x; c < width; c += blockDim.x) dst[c] = to_f32<T>(src[c]) + to_f32<T>(ps[c]);
+    for (int c = threadIdx.x; c < width; c += blockDim.x) dst[c] = fmaf(to_f32<T>(src[c]), scale, to_f32<T>(ps[c]));
     return;
   }
-  for (int c = threadIdx.x; c < width; c += blockDim.x) dst[c] = to_f32<T>(src[c]);
+  for (int c = threadIdx.x; c < width; c += blockDim.x) dst[c] = to_f32<T>(src[c]) * scale;
 }
 
 __device__ __forceinline__ void embed_unpack8(const uint4 raw, float4& lo, float4& hi) {
@@ -50,7 +50,8 @@ __device__ __forceinline__ void embed_unpack8(const uint4 raw, float4& lo, float
 // eight elements per thread, no loop (bfloat16 tables whose width is a multiple of 8)
 __global__ void embed_bf16x8_kernel(const int32_t* __restrict__ ids, const bf16_t* __restrict__ table,
                                     float* __restrict__ out, int width, int vocab, size_t total_vec,
-                                    const int32_t* __restrict__ positions, const bf16_t* __restrict__ pos_table, int pos_rows) {
+                                    const int32_t* __restrict__ positions, const bf16_t* __restrict__ pos_table, int pos_rows,
+                                    float scale) {
   const size_t v = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x;
   if (v >= total_vec) return;
   const int per_row = width / 8;
@@ -60,6 +61,10 @@ __global__ void embed_bf16x8_kernel(const int32_t* __restrict__ ids, const bf16_
   id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
   float4 lo, hi;
   embed_unpack8(*reinterpret_cast<const uint4*>(table + static_cast<size_t>(id) * width + c), lo, hi);
+  if (scale != 1.f) {  // (the token's row alone is scaled)
+    lo.x *= scale; lo.y *= scale; lo.z *= scale; lo.w *= scale;
+    hi.x *= scale; hi.y *= scale; hi.z *= scale; hi.w *= scale;
+  }
   if (pos_table != nullptr) {
     int p = positions[n];
     p = p < 0 ? 0 : (p >= pos_rows ? pos_rows - 1 : p);
@@ -73,10 +78,11 @@ __global__ void embed_bf16x8_kernel(const int32_t* __restrict__ ids, const bf16_
   *reinterpret_cast<float4*>(dst + 4) = hi;
 }
 
-// positions / pos_table (of the table's dtype, pos_rows rows) null: the token's row alone
+// positions / pos_table (of the table's dtype, pos_rows rows) null: the token's row alone; scale: what the
+// token's row is multiplied with in float32 (1: nothing)
 extern "C" int yk_embed(const int32_t* ids, const void* table, int table_dtype, float* out,
                         int n_tokens, int width, int vocab, const int32_t* positions, const void* pos_table, int pos_rows,
-                        hipStream_t stream) {
+                        float scale, hipStream_t stream) {
   YK_REQUIRE(n_tokens >= 0 && width > 0 && vocab > 0, "embed: bad sizes");
   YK_REQUIRE(pos_table == nullptr || (positions != nullptr && pos_rows > 0), "embed: a position table needs positions");
   if (n_tokens == 0) return 0;
@@ -85,16 +91,16 @@ extern "C" int yk_embed(const int32_t* ids, const void* table, int table_dtype, 
     const size_t total_vec = static_cast<size_t>(n_tokens) * (width / 8);
     embed_bf16x8_kernel<<<static_cast<unsigned>((total_vec + 255) / 256), 256, 0, stream>>>(
         ids, static_cast<const bf16_t*>(table), out, width, vocab, total_vec, positions, static_cast<const bf16_t*>(pos_table),
-        pos_rows);
+        pos_rows, scale);
     return yk_check_launch("embed");
   }
   dim3 grid(n_tokens), block(256);
   if (table_dtype == YK_F32)
     embed_kernel<float><<<grid, block, 0, stream>>>(ids, static_cast<const float*>(table), out, width, vocab, positions,
-                                                    static_cast<const float*>(pos_table), pos_rows);
+                                                    static_cast<const float*>(pos_table), pos_rows, scale);
   else if (table_dtype == YK_BF16)
     embed_kernel<bf16_t><<<grid, block, 0, stream>>>(ids, static_cast<const bf16_t*>(table), out, width, vocab, positions,
-                                                     static_cast<const bf16_t*>(pos_table), pos_rows);
+                                                     static_cast<const bf16_t*>(pos_table), pos_rows, scale);
   else
     return yk_fail("embed: unsupported table dtype");
   return yk_check_launch("embed");
@@ -157,7 +163,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ residual, const TD* __res
                                    int n_splits, size_t split_stride, int round_sum,
                                    const int32_t* __restrict__ rows, const TW* __restrict__ weight,
                                    TO* __restrict__ out, int width, float eps, int unit_offset,
-                                   const int32_t* __restrict__ table_ids, int table_rows) {
+                                   const int32_t* __restrict__ table_ids, int table_rows, const float* __restrict__ add_row) {
   __shared__ float scratch[17];
   const int r = blockIdx.x;
   const size_t src = rows ? static_cast<size_t>(rows[r]) : static_cast<size_t>(r);
@@ -171,8 +177,9 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ residual, const TD* __res
       float d = 0.f;
       for (int s = 0; s < n_splits; ++s) d += to_f32<TD>(del[s * split_stride + c]);
       v += as_output(d, round_sum);
-      if (!rows && res) res[c] = v;
     }
+    if (add_row) v += add_row[c];
+    if ((del || add_row) && !rows && res) res[c] = v;
     ss += v * v;
   }
   ss = block_sum(ss, scratch);
@@ -199,7 +206,8 @@ template <typename TD, typename TW, typename TO, int NORM_IT>
 __global__ __launch_bounds__(1024) void add_rmsnorm_vec_kernel(
     float* __restrict__ residual, const TD* __restrict__ delta, int n_splits, size_t split_stride,
     int round_sum, const int32_t* __restrict__ rows, const TW* __restrict__ weight, TO* __restrict__ out,
-    int width, float eps, int unit_offset, const int32_t* __restrict__ table_ids, int table_rows) {
+    int width, float eps, int unit_offset, const int32_t* __restrict__ table_ids, int table_rows,
+    const float* __restrict__ add_row) {
   __shared__ float scratch[17];
   const int r = blockIdx.x;
   const size_t src = rows ? static_cast<size_t>(rows[r]) : static_cast<size_t>(r);
@@ -256,7 +264,14 @@ __global__ __launch_bounds__(1024) void add_rmsnorm_vec_kernel(
   for (int it = 0; it < NORM_IT; ++it) {
     const int c = (threadIdx.x + it * blockDim.x) * 4;
     if (c < width) {
-      if (del && !rows && res) store4<float>(res + c, v[it]);
+      if (add_row) {  // one vector for every row (the launcher allows it only where the residual is written back)
+        const float4 a = load4<float>(add_row + c);
+        v[it].x += a.x;
+        v[it].y += a.y;
+        v[it].z += a.z;
+        v[it].w += a.w;
+      }
+      if ((del || add_row) && !rows && res) store4<float>(res + c, v[it]);
       ss += v[it].x * v[it].x + v[it].y * v[it].y + v[it].z * v[it].z + v[it].w * v[it].w;
     }
   }
@@ -282,8 +297,8 @@ template <typename TD, typename TW, typename TO>
 static int launch_add_rmsnorm(float* residual, const void* delta, int n_splits, size_t split_stride,
                               int round_sum, const int32_t* rows, const void* weight, void* out, int n_rows,
                               int width, float eps, int unit_offset, const int32_t* table_ids, int table_rows,
-                              hipStream_t stream) {
-  const bool aligned = width % 4 == 0 && reinterpret_cast<uintptr_t>(residual) % 16 == 0 &&
+                              const float* add_row, hipStream_t stream) {
+  const bool aligned = width % 4 == 0 && reinterpret_cast<uintptr_t>(residual) % 16 == 0 && reinterpret_cast<uintptr_t>(add_row) % 16 == 0 &&
                        reinterpret_cast<uintptr_t>(delta) % 16 == 0 && reinterpret_cast<uintptr_t>(weight) % 16 == 0 &&
                        reinterpret_cast<uintptr_t>(out) % 16 == 0 && split_stride % 4 == 0;
   if (aligned && width <= 4 * NORM_IT_MAX * 512) {
@@ -297,7 +312,7 @@ static int launch_add_rmsnorm(float* residual, const void* delta, int n_splits, 
 #define YK_NORM(IT)                                                                           \
     add_rmsnorm_vec_kernel<TD, TW, TO, IT><<<n_rows, threads, 0, stream>>>(                   \
         residual, static_cast<const TD*>(delta), n_splits, split_stride, round_sum, rows,     \
-        static_cast<const TW*>(weight), static_cast<TO*>(out), width, eps, unit_offset, table_ids, table_rows)
+        static_cast<const TW*>(weight), static_cast<TO*>(out), width, eps, unit_offset, table_ids, table_rows, add_row)
     if (pieces <= 1) YK_NORM(1);
     else if (pieces <= 2) YK_NORM(2);
     else if (pieces <= 4) YK_NORM(4);
@@ -306,7 +321,7 @@ static int launch_add_rmsnorm(float* residual, const void* delta, int n_splits, 
   } else {
     add_rmsnorm_kernel<TD, TW, TO><<<n_rows, width >= 2048 ? 512 : 256, 0, stream>>>(
         residual, static_cast<const TD*>(delta), n_splits, split_stride, round_sum, rows,
-        static_cast<const TW*>(weight), static_cast<TO*>(out), width, eps, unit_offset, table_ids, table_rows);
+        static_cast<const TW*>(weight), static_cast<TO*>(out), width, eps, unit_offset, table_ids, table_rows, add_row);
   }
   return yk_check_launch("add_rmsnorm");
 }
@@ -315,11 +330,14 @@ static int launch_add_rmsnorm(float* residual, const void* delta, int n_splits, 
 // float32 delta laid out [n_splits][rows of the residual][width]; round_sum: the slices' sum
 // is rounded to bfloat16 before it is added.  table_ids (null, or one id per residual row):
 // delta is an embedding table of table_rows rows and the residual starts as its rows
-// table_ids[.] (n_splits 1, no rows).
+// table_ids[.] (n_splits 1, no rows).  add_row (null, or float32 [width]): one vector that every row of the residual
+// receives as well (no rows: the residual is written back).
 extern "C" int yk_add_rmsnorm(float* residual, const void* delta, int delta_dtype, int n_splits,
                               int round_sum, const int32_t* rows, const void* weight, int weight_dtype, void* out,
                               int out_dtype, int n_rows, int n_residual_rows, int width, float eps,
-                              int unit_offset, const int32_t* table_ids, int table_rows, hipStream_t stream) {
+                              int unit_offset, const int32_t* table_ids, int table_rows, const float* add_row,
+                              hipStream_t stream) {
+  YK_REQUIRE(!add_row || (residual && !rows), "add_rmsnorm: a vector for every row joins a residual that is written back");
   YK_REQUIRE(n_rows >= 0 && width > 0 && n_residual_rows >= 0, "add_rmsnorm: bad sizes");
   YK_REQUIRE(residual || (delta && !table_ids), "add_rmsnorm: without a residual there must be rows to normalise");
   YK_REQUIRE(!table_ids || (delta && n_splits == 1 && !rows && table_rows > 0 && !round_sum),
@@ -335,7 +353,7 @@ extern "C" int yk_add_rmsnorm(float* residual, const void* delta, int delta_dtyp
   const size_t stride = static_cast<size_t>(n_residual_rows) * width;
 #define YK_CASE(DD, TD, WD, TW, OD, TO)                                  \
   if (delta_dtype == DD && weight_dtype == WD && out_dtype == OD)        \
-    return launch_add_rmsnorm<TD, TW, TO>(residual, delta, n_splits, stride, round_sum, rows, weight, out, n_rows, width, eps, unit_offset, table_ids, table_rows, stream);
+    return launch_add_rmsnorm<TD, TW, TO>(residual, delta, n_splits, stride, round_sum, rows, weight, out, n_rows, width, eps, unit_offset, table_ids, table_rows, add_row, stream);
   YK_CASE(YK_F32, float, YK_F32, float, YK_F32, float)
   YK_CASE(YK_F32, float, YK_F32, float, YK_BF16, bf16_t)
   YK_CASE(YK_F32, float, YK_BF16, bf16_t, YK_F32, float)

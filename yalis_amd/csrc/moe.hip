@@ -96,11 +96,14 @@ extern "C" int yk_moe_route(const int32_t* token_ids, const int32_t* table, int 
 // Per token: the `top` experts with the largest logits (ties: the lower number), their numbers into choice
 // [tokens][top], and the token's row once per chosen expert, multiplied by that expert's score sigmoid(logit), into xs
 // [tokens * top][hidden]: the score weighs what the expert reads, not what it returns.  A workgroup a token; its
-// first wave chooses.
+// first wave chooses.  bias [n_experts] (or null) joins the logits before the choice.  With `weights` (float32 [tokens][top])
+// in place of xs, the chosen experts' weights are written instead: the softmax over the chosen logits alone (they weigh
+// what the experts return; nothing is copied).
 template <typename T>
 __global__ __launch_bounds__(256) void moe_router_topk_kernel(const float* __restrict__ logits, int logits_stride, int n_experts, int top,
                                                               const T* __restrict__ x, int x_stride, int hidden,
-                                                              int32_t* __restrict__ choice, T* __restrict__ xs) {
+                                                              int32_t* __restrict__ choice, T* __restrict__ xs,
+                                                              const float* __restrict__ bias, float* __restrict__ weights) {
   extern __shared__ float sel[];  // [top] scores, then [top] numbers (as ints)
   int* sel_e = reinterpret_cast<int*>(sel + top);
   const int n = blockIdx.x, lane = threadIdx.x;
@@ -112,7 +115,7 @@ __global__ __launch_bounds__(256) void moe_router_topk_kernel(const float* __res
       for (int e = lane; e < n_experts; e += kWave) {
         bool taken = false;
         for (int j = 0; j < k; ++j) taken |= sel_e[j] == e;
-        const float v = row[e];
+        const float v = bias != nullptr ? row[e] + bias[e] : row[e];
         // (a NaN is never larger: such a row falls back on the lowest free numbers)
         if (!taken && (v > best || (best_e == 0x7fffffff) || (v == best && e < best_e))) {
           best = v;
@@ -130,13 +133,19 @@ __global__ __launch_bounds__(256) void moe_router_topk_kernel(const float* __res
       }
       if (lane == 0) {
         sel_e[k] = best_e;
-        sel[k] = 1.f / (1.f + expf(-best));
+        sel[k] = weights != nullptr ? best : 1.f / (1.f + expf(-best));
         choice[static_cast<size_t>(n) * top + k] = best_e;
       }
       __builtin_amdgcn_wave_barrier();
       __threadfence_block();
     }
+    if (weights != nullptr && lane == 0) {  // sel[0] is the largest
+      float sum = 0.f;
+      for (int k = 0; k < top; ++k) sum += expf(sel[k] - sel[0]);
+      for (int k = 0; k < top; ++k) weights[static_cast<size_t>(n) * top + k] = expf(sel[k] - sel[0]) / sum;
+    }
   }
+  if (weights != nullptr) return;
   __syncthreads();
   const T* src = x + static_cast<size_t>(n) * x_stride;
   for (int c = threadIdx.x; c < hidden; c += blockDim.x) {
@@ -146,29 +155,35 @@ __global__ __launch_bounds__(256) void moe_router_topk_kernel(const float* __res
 }
 
 extern "C" int yk_moe_router_topk(const float* logits, int logits_stride, int n_experts, int top, const void* x, int x_stride, int dtype,
-                                  int hidden, int32_t* choice, void* xs, int n_tokens, hipStream_t stream) {
-  YK_REQUIRE(n_tokens >= 0 && n_experts >= 1 && top >= 1 && top <= n_experts && top <= 64 && hidden > 0 && x_stride >= hidden &&
-                 logits_stride >= n_experts,
+                                  int hidden, int32_t* choice, void* xs, int n_tokens, const float* bias, float* weights,
+                                  hipStream_t stream) {
+  YK_REQUIRE(n_tokens >= 0 && n_experts >= 1 && top >= 1 && top <= n_experts && top <= 64 && logits_stride >= n_experts,
              "moe_router_topk: bad sizes (up to 64 experts a token)");
+  YK_REQUIRE((weights != nullptr) != (xs != nullptr), "moe_router_topk: weights for the outputs, or scaled copies of the inputs");
+  YK_REQUIRE(weights != nullptr || (x != nullptr && hidden > 0 && x_stride >= hidden), "moe_router_topk: bad input rows");
   if (n_tokens == 0) return 0;
   const size_t lds = 2 * static_cast<size_t>(top) * sizeof(float);
-  if (dtype == YK_F32)
+  if (weights != nullptr)  // one wave chooses and weighs; there is nothing to copy
+    moe_router_topk_kernel<float><<<n_tokens, 64, lds, stream>>>(logits, logits_stride, n_experts, top, nullptr, 0, 0, choice, nullptr, bias,
+                                                                 weights);
+  else if (dtype == YK_F32)
     moe_router_topk_kernel<float><<<n_tokens, 256, lds, stream>>>(logits, logits_stride, n_experts, top, static_cast<const float*>(x), x_stride,
-                                                                  hidden, choice, static_cast<float*>(xs));
+                                                                  hidden, choice, static_cast<float*>(xs), bias, nullptr);
   else if (dtype == YK_BF16)
     moe_router_topk_kernel<bf16_t><<<n_tokens, 256, lds, stream>>>(logits, logits_stride, n_experts, top, static_cast<const bf16_t*>(x), x_stride,
-                                                                   hidden, choice, static_cast<bf16_t*>(xs));
+                                                                   hidden, choice, static_cast<bf16_t*>(xs), bias, nullptr);
   else
     return yk_fail("moe_router_topk: unsupported dtype");
   return yk_check_launch("moe_router_topk");
 }
 
 // out[n, :] = dense[n, :] (a tensor, a product's unreduced slices, or nothing) + weight * the sum of the token's `top`
-// rows of rows [tokens * top][width]: what a mixture adds to the stream, as one float32 tensor
+// rows of rows [tokens * top][width] (each times its own entry of row_weights [tokens * top] where given): what a mixture adds to
+// the stream, as one float32 tensor
 template <typename TD>
 __global__ void moe_combine_kernel(const TD* __restrict__ dense, int n_splits, size_t split_stride, int round_sum,
                                    const float* __restrict__ rows, int top, float weight, float* __restrict__ out, int width,
-                                   size_t total) {
+                                   size_t total, const float* __restrict__ row_weights) {
   for (size_t i = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; i < total;
        i += static_cast<size_t>(gridDim.x) * blockDim.x) {
     const size_t n = i / width;
@@ -179,23 +194,26 @@ __global__ void moe_combine_kernel(const TD* __restrict__ dense, int n_splits, s
       d = as_output(d, round_sum);
     }
     float e = 0.f;
-    for (int k = 0; k < top; ++k) e += rows[(n * top + k) * width + c];
+    if (row_weights != nullptr)  // every row has a weight of its own
+      for (int k = 0; k < top; ++k) e = fmaf(row_weights[n * top + k], rows[(n * top + k) * width + c], e);
+    else
+      for (int k = 0; k < top; ++k) e += rows[(n * top + k) * width + c];
     out[i] = fmaf(weight, e, d);
   }
 }
 
 extern "C" int yk_moe_combine(const void* dense, int dense_dtype, int n_splits, int round_sum, const float* rows, int top,
-                              float weight, float* out, int n_tokens, int width, hipStream_t stream) {
+                              float weight, float* out, int n_tokens, int width, const float* row_weights, hipStream_t stream) {
   YK_REQUIRE(n_tokens >= 0 && width > 0 && top >= 1 && n_splits >= 1 && (n_splits == 1 || dense_dtype == YK_F32), "moe_combine: bad sizes");
   if (n_tokens == 0) return 0;
   const size_t total = static_cast<size_t>(n_tokens) * width;
   const int grid = static_cast<int>(std::min<size_t>((total + 255) / 256, 1 << 20));
   if (dense == nullptr || dense_dtype == YK_F32)
     moe_combine_kernel<float><<<grid, 256, 0, stream>>>(static_cast<const float*>(dense), n_splits, total, round_sum, rows, top,
-                                                        weight, out, width, total);
+                                                        weight, out, width, total, row_weights);
   else if (dense_dtype == YK_BF16)
     moe_combine_kernel<bf16_t><<<grid, 256, 0, stream>>>(static_cast<const bf16_t*>(dense), n_splits, total, round_sum, rows, top,
-                                                         weight, out, width, total);
+                                                         weight, out, width, total, row_weights);
   else
     return yk_fail("moe_combine: unsupported dtype");
   return yk_check_launch("moe_combine");
@@ -206,12 +224,21 @@ template <typename T, typename TW>
 __global__ __launch_bounds__(256) void moe_gate_up_fma_kernel(
     const T* __restrict__ x, int x_stride, const TW* __restrict__ w, const int32_t* __restrict__ order,
     const int32_t* __restrict__ slot_expert, int top, int hidden, int ff, int kind, float p0, float p1,
-    T* __restrict__ y) {
+    T* __restrict__ y, int gated) {
   extern __shared__ float xs[];  // [hidden]
   const int i = blockIdx.x;
   const int token = order[i] / top, e = slot_expert[i];
   for (int k = threadIdx.x; k < hidden; k += blockDim.x) xs[k] = to_f32<T>(x[static_cast<size_t>(token) * x_stride + k]);
   __syncthreads();
+  if (!gated) {  // an expert without a gate: act(up x), the weights [experts][ff][hidden]
+    for (int j = blockIdx.y * blockDim.x + threadIdx.x; j < ff; j += gridDim.y * blockDim.x) {
+      const TW* wu = w + (static_cast<size_t>(e) * ff + j) * hidden;
+      float u = 0.f;
+      for (int k = 0; k < hidden; ++k) u = fmaf(to_f32<TW>(wu[k]), xs[k], u);
+      y[static_cast<size_t>(i) * ff + j] = from_f32<T>(act_plain(u, kind));
+    }
+    return;
+  }
   for (int j = blockIdx.y * blockDim.x + threadIdx.x; j < ff; j += gridDim.y * blockDim.x) {
     const TW* wg = w + (static_cast<size_t>(e) * 2 * ff + j) * hidden;
     const TW* wu = wg + static_cast<size_t>(ff) * hidden;
@@ -270,7 +297,9 @@ __device__ __forceinline__ void moe_tile_of(int n_groups, int& tile, int& group)
 // KS: the four waves of a workgroup share one set of features and divide K between them (their
 // sums meet in LDS): steps of few pairs have few tiles, and this way four times the waves pull on
 // an expert's weights.
-template <int MT, int FT, int WR, bool KS>
+// GATED false: experts without a gate, act(up x) with a plain activation; the weights are [experts][ff][hidden] and only
+// the `u` half of everything below is computed.
+template <int MT, int FT, int WR, bool KS, bool GATED>
 __global__ __launch_bounds__(256 * WR) void moe_gate_up_mfma_kernel(
     const bf16_t* __restrict__ x, int x_stride, const bf16_t* __restrict__ w, const int32_t* __restrict__ order,
     const int32_t* __restrict__ tiles, const int32_t* __restrict__ n_tiles, int top, int hidden, int ff, int kind,
@@ -289,8 +318,8 @@ __global__ __launch_bounds__(256 * WR) void moe_gate_up_mfma_kernel(
 #pragma unroll
   for (int f = 0; f < FT; ++f) {
     const int row = min(f0 + 16 * f + r, ff - 1);  // (tiles beyond the width repeat its last row and are not stored)
-    wg[f] = w + (static_cast<size_t>(e) * 2 * ff + row) * hidden + 8 * g;
-    wu[f] = wg[f] + static_cast<size_t>(ff) * hidden;
+    wg[f] = w + (static_cast<size_t>(e) * (GATED ? 2 : 1) * ff + row) * hidden + 8 * g;
+    wu[f] = GATED ? wg[f] + static_cast<size_t>(ff) * hidden : wg[f];
   }
   const bf16_t* xr[MT];
 #pragma unroll
@@ -307,7 +336,7 @@ __global__ __launch_bounds__(256 * WR) void moe_gate_up_mfma_kernel(
 #define MOE_LOAD(A, B, K0)                                                                  \
   {                                                                                         \
     _Pragma("unroll") for (int f = 0; f < FT; ++f) {                                        \
-      A[0][f].u = *reinterpret_cast<const u32x4_t*>(wg[f] + (K0));                          \
+      if (GATED) A[0][f].u = *reinterpret_cast<const u32x4_t*>(wg[f] + (K0));               \
       A[1][f].u = *reinterpret_cast<const u32x4_t*>(wu[f] + (K0));                          \
     }                                                                                       \
     _Pragma("unroll") for (int m = 0; m < MT; ++m) B[m].u = *reinterpret_cast<const u32x4_t*>(xr[m] + (K0)); \
@@ -316,7 +345,7 @@ __global__ __launch_bounds__(256 * WR) void moe_gate_up_mfma_kernel(
   {                                                                                         \
     _Pragma("unroll") for (int f = 0; f < FT; ++f)                                          \
     _Pragma("unroll") for (int m = 0; m < MT; ++m) {                                        \
-      ag[f][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A[0][f].v, B[m].v, ag[f][m], 0, 0, 0); \
+      if (GATED) ag[f][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A[0][f].v, B[m].v, ag[f][m], 0, 0, 0); \
       au[f][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A[1][f].v, B[m].v, au[f][m], 0, 0, 0); \
     }                                                                                       \
   }
@@ -337,7 +366,7 @@ __global__ __launch_bounds__(256 * WR) void moe_gate_up_mfma_kernel(
       for (int f = 0; f < FT; ++f)
 #pragma unroll
         for (int m = 0; m < MT; ++m) {
-          part[wave - 1][(2 * f) * MT + m][lane] = ag[f][m];
+          if (GATED) part[wave - 1][(2 * f) * MT + m][lane] = ag[f][m];
           part[wave - 1][(2 * f + 1) * MT + m][lane] = au[f][m];
         }
     }
@@ -349,7 +378,7 @@ __global__ __launch_bounds__(256 * WR) void moe_gate_up_mfma_kernel(
       for (int f = 0; f < FT; ++f)
 #pragma unroll
         for (int m = 0; m < MT; ++m) {
-          ag[f][m] += part[w2][(2 * f) * MT + m][lane];
+          if (GATED) ag[f][m] += part[w2][(2 * f) * MT + m][lane];
           au[f][m] += part[w2][(2 * f + 1) * MT + m][lane];
         }
   }
@@ -360,8 +389,13 @@ __global__ __launch_bounds__(256 * WR) void moe_gate_up_mfma_kernel(
     for (int m = 0; m < MT; ++m) {
       if (16 * m + r < count) {
         uint32_t o[2];
-        o[0] = pack_bf16x2(gated_pair(ag[f][m][0], au[f][m][0], kind, p0, p1), gated_pair(ag[f][m][1], au[f][m][1], kind, p0, p1));
-        o[1] = pack_bf16x2(gated_pair(ag[f][m][2], au[f][m][2], kind, p0, p1), gated_pair(ag[f][m][3], au[f][m][3], kind, p0, p1));
+        if (GATED) {
+          o[0] = pack_bf16x2(gated_pair(ag[f][m][0], au[f][m][0], kind, p0, p1), gated_pair(ag[f][m][1], au[f][m][1], kind, p0, p1));
+          o[1] = pack_bf16x2(gated_pair(ag[f][m][2], au[f][m][2], kind, p0, p1), gated_pair(ag[f][m][3], au[f][m][3], kind, p0, p1));
+        } else {
+          o[0] = pack_bf16x2(act_plain(au[f][m][0], kind), act_plain(au[f][m][1], kind));
+          o[1] = pack_bf16x2(act_plain(au[f][m][2], kind), act_plain(au[f][m][3], kind));
+        }
         *reinterpret_cast<uint2*>(y + static_cast<size_t>(first + 16 * m + r) * ff + f0 + 16 * f + 4 * g) = make_uint2(o[0], o[1]);
       }
     }
@@ -458,9 +492,9 @@ static bool aligned16(const void* p) { return reinterpret_cast<uintptr_t>(p) % 1
 extern "C" int yk_moe_gate_up(const void* x, int x_stride, int dtype, const void* w, int w_dtype, const int32_t* order,
                               const int32_t* slot_expert, const int32_t* tiles, const int32_t* n_tiles, int tile_rows,
                               int max_tiles, int n_pairs, int top, int hidden, int ff, int kind, float p0, float p1,
-                              void* y, hipStream_t stream) {
+                              void* y, int gated, hipStream_t stream) {
   YK_REQUIRE(n_pairs >= 0 && top >= 1 && hidden > 0 && ff > 0 && x_stride >= hidden, "moe_gate_up: bad sizes");
-  YK_REQUIRE(kind >= 0 && kind < YK_GATED_KINDS, "moe_gate_up: unknown activation");
+  YK_REQUIRE(kind >= 0 && kind < (gated ? YK_GATED_KINDS : YK_PLAIN_KINDS), "moe_gate_up: unknown activation");
   if (n_pairs == 0) return 0;
   if (dtype == YK_BF16 && w_dtype == YK_BF16 && yk_moe_mfma_ok(hidden, ff, x_stride) && aligned16(x) && aligned16(w) &&
       aligned16(y) && (tile_rows == 16 || tile_rows == 64 || tile_rows == 128)) {
@@ -470,12 +504,17 @@ extern "C" int yk_moe_gate_up(const void* x, int x_stride, int dtype, const void
     YK_REQUIRE(n_wg <= 0x7fffffffLL, "moe_gate_up: too many tiles for one launch");
     dim3 grid(static_cast<unsigned>(n_wg));
 #define YK_MOE_GU(MT, WR, KS)                                                                                   \
-  moe_gate_up_mfma_kernel<MT, FT, WR, KS><<<grid, 256 * WR, 0, stream>>>(                                            \
-      static_cast<const bf16_t*>(x), x_stride, static_cast<const bf16_t*>(w), order, tiles, n_tiles, top, hidden, ff, \
-      kind, p0, p1, static_cast<bf16_t*>(y), n_groups)
-    if (tile_rows == 16) YK_MOE_GU(1, 1, true);
-    else if (tile_rows == 64) YK_MOE_GU(4, 1, false);
-    else YK_MOE_GU(4, 2, false);
+  if (gated)                                                                                                     \
+    moe_gate_up_mfma_kernel<MT, FT, WR, KS, true><<<grid, 256 * WR, 0, stream>>>(                                     \
+        static_cast<const bf16_t*>(x), x_stride, static_cast<const bf16_t*>(w), order, tiles, n_tiles, top, hidden, ff, \
+        kind, p0, p1, static_cast<bf16_t*>(y), n_groups);                                                         \
+  else                                                                                                           \
+    moe_gate_up_mfma_kernel<MT, FT, WR, KS, false><<<grid, 256 * WR, 0, stream>>>(                                    \
+        static_cast<const bf16_t*>(x), x_stride, static_cast<const bf16_t*>(w), order, tiles, n_tiles, top, hidden, ff, \
+        kind, p0, p1, static_cast<bf16_t*>(y), n_groups)
+    if (tile_rows == 16) { YK_MOE_GU(1, 1, true); }
+    else if (tile_rows == 64) { YK_MOE_GU(4, 1, false); }
+    else { YK_MOE_GU(4, 2, false); }
 #undef YK_MOE_GU
     return yk_check_launch("moe_gate_up (matrix cores)");
   }
@@ -486,7 +525,7 @@ extern "C" int yk_moe_gate_up(const void* x, int x_stride, int dtype, const void
   if (dtype == D && w_dtype == WD) {                                                                               \
     moe_gate_up_fma_kernel<T, TW><<<grid, block, lds, stream>>>(static_cast<const T*>(x), x_stride, static_cast<const TW*>(w), \
                                                                 order, slot_expert, top, hidden, ff, kind, p0, p1,            \
-                                                                static_cast<T*>(y));                                          \
+                                                                static_cast<T*>(y), gated);                                   \
     return yk_check_launch("moe_gate_up");                                                                         \
   }
   YK_CASE(YK_F32, float, YK_F32, float)

@@ -163,7 +163,7 @@ class DecoderModel:
         """Every part takes its tensors from ``tensors``: a dict, or a source that makes
         each tensor when it is asked for (each part asks once for each of its names)."""
         for name in self.added_tables:
-            self._added[name] = tensors[name].contiguous()
+            self._added[name] = tensors[name].to(torch.float32).contiguous()  # (what the stream is summed in)
         for p in self.all_parts():
             p.load(tensors)
 

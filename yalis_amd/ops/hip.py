@@ -48,9 +48,9 @@ def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
 _SIGNATURES = {
     "yk_abi_version": ([], _c_int),
     "yk_cache_tiled": ([_c_int, _c_int, _c_int], _c_int),
-    "yk_embed": ([_vp, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _vp, _vp, _c_int, _vp], _c_int),
+    "yk_embed": ([_vp, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _vp, _vp, _c_int, _c_float, _vp], _c_int),
     "yk_add_rmsnorm": (
-        [_vp, _vp, _c_int, _c_int, _c_int, _vp, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _vp, _c_int, _vp],
+        [_vp, _vp, _c_int, _c_int, _c_int, _vp, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _vp, _c_int, _vp, _vp],
         _c_int,
     ),
     "yk_rope_append": (
@@ -68,13 +68,17 @@ _SIGNATURES = {
     "yk_qkv_prepare": (
         [_vp, _c_int, _c_int, _c_int, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _vp, _vp, _c_int,
          _c_int, _c_float, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _c_float, _vp, _vp, _c_int, _c_int, _vp, _vp, _vp, _c_int,
-         _c_int, _vp],
+         _c_int, _vp, _vp, _c_int, _vp],
+        _c_int,
+    ),
+    "yk_qk_row_scales": (
+        [_vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _c_int, _c_float, _vp, _c_float, _c_int, _vp, _vp],
         _c_int,
     ),
     "yk_attn_masked": (
         [_vp, _c_int, _vp, _vp, _vp, _c_int, _vp, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float,
          _c_float, _c_int, _c_int, _c_int, _vp, _vp, _c_int, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _vp,
-         _c_int, _vp],
+         _c_int, _vp, _vp],
         _c_int,
     ),
     "yk_attn_finish": (
@@ -134,12 +138,12 @@ _SIGNATURES = {
     "yk_rglru_scan": ([_vp, _vp, _vp, _c_int, _vp, _c_int, _c_int, _vp, _vp, _vp, _vp, _vp, _vp, _c_int, _c_int, _c_int, _vp], _c_int),
     "yk_moe_max_tiles": ([_c_int, _c_int, _c_int], _c_int),
     "yk_moe_mfma_ok": ([_c_int, _c_int, _c_int], _c_int),
-    "yk_moe_router_topk": ([_vp, _c_int, _c_int, _c_int, _vp, _c_int, _c_int, _c_int, _vp, _vp, _c_int, _vp], _c_int),
-    "yk_moe_combine": ([_vp, _c_int, _c_int, _c_int, _vp, _c_int, _c_float, _vp, _c_int, _c_int, _vp], _c_int),
+    "yk_moe_router_topk": ([_vp, _c_int, _c_int, _c_int, _vp, _c_int, _c_int, _c_int, _vp, _vp, _c_int, _vp, _vp, _vp], _c_int),
+    "yk_moe_combine": ([_vp, _c_int, _c_int, _c_int, _vp, _c_int, _c_float, _vp, _c_int, _c_int, _vp, _vp], _c_int),
     "yk_moe_route": ([_vp, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _vp, _vp, _vp, _vp], _c_int),
     "yk_moe_gate_up": (
         [_vp, _c_int, _c_int, _vp, _c_int, _vp, _vp, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float,
-         _c_float, _vp, _vp],
+         _c_float, _vp, _c_int, _vp],
         _c_int,
     ),
     "yk_moe_down": ([_vp, _c_int, _vp, _c_int, _vp, _vp, _vp, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _vp, _vp], _c_int),
@@ -209,7 +213,7 @@ _LATER_SIGNATURES = {
         "yk_probe_mfma_bf16": ([_c_int, _c_int, _vp, _vp], _c_int),
     },
 }
-_ABI = 20
+_ABI = 21
 
 # Rows of x up to which the hand-written matrix-core kernel runs a bfloat16 product;
 # above it the vendor library does.
@@ -483,8 +487,8 @@ class HipOps:
         return 2 if workgroups >= 1024 or fewest_keys >= 1024 else 1
 
     # ------------------------------------------------------------------ embedding
-    def embed(self, token_ids: torch.Tensor, table: torch.Tensor, positions=None, position_table=None) -> torch.Tensor:
-        """float32 rows table[id] (+ position_table[position], a learned vector per absolute position, summed in
+    def embed(self, token_ids: torch.Tensor, table: torch.Tensor, positions=None, position_table=None, scale: float = 1.0) -> torch.Tensor:
+        """float32 rows table[id] * scale (+ position_table[position], a learned vector per absolute position, summed in
         float32)."""
         self._rows(table, "embed table")
         n = token_ids.numel()
@@ -498,7 +502,7 @@ class HipOps:
             self.lib.yk_embed(
                 token_ids.data_ptr(), table.data_ptr(), _code(table.dtype), out.data_ptr(), n,
                 table.shape[1], table.shape[0], _ptr(positions) if position_table is not None else None, _ptr(position_table),
-                0 if position_table is None else position_table.shape[0], self._stream(),
+                0 if position_table is None else position_table.shape[0], float(scale), self._stream(),
             )
         )
         return out
@@ -531,13 +535,15 @@ class HipOps:
         self._check(
             self.lib.yk_add_rmsnorm(
                 None, src.data_ptr(), _code(src.dtype), n_splits, round_sum, None, weight.data_ptr(), _code(weight.dtype),
-                out.data_ptr(), _code(out_dtype), n, n, width, float(eps), int(bool(unit_offset)), None, 0, self._stream(),
+                out.data_ptr(), _code(out_dtype), n, n, width, float(eps), int(bool(unit_offset)), None, 0, None, self._stream(),
             )
         )
         return out
 
-    def _norm(self, residual, delta, rows, weight, eps, unit_offset, out_dtype, n_out):
+    def _norm(self, residual, delta, rows, weight, eps, unit_offset, out_dtype, n_out, row=None):
         self._rows(residual, "residual")
+        if row is not None and (rows is not None or row.dtype != torch.float32 or row.numel() != residual.shape[1] or not row.is_contiguous()):
+            raise KernelError("add_rmsnorm: the vector for every token is contiguous float32 [width], and the residual is written back")
         if residual.dtype != torch.float32 or not residual.is_contiguous():
             raise KernelError("the residual stream must be contiguous float32")
         width = residual.shape[1]
@@ -565,14 +571,16 @@ class HipOps:
             self.lib.yk_add_rmsnorm(
                 residual.data_ptr(), _ptr(delta), 0 if delta is None else _code(delta.dtype), n_splits, round_sum,
                 _ptr(rows), weight.data_ptr(), _code(weight.dtype), out.data_ptr(), _code(out_dtype),
-                n_out, residual.shape[0], width, float(eps), int(bool(unit_offset)), _ptr(table_ids), table_rows,
+                n_out, residual.shape[0], width, float(eps), int(bool(unit_offset)), _ptr(table_ids), table_rows, _ptr(row),
                 self._stream(),
             )
         )
         return out
 
-    def add_rmsnorm(self, residual, delta, weight, eps, unit_offset, out_dtype):
-        return self._norm(residual, delta, None, weight, eps, unit_offset, out_dtype, residual.shape[0])
+    def add_rmsnorm(self, residual, delta, weight, eps, unit_offset, out_dtype, row=None):
+        """residual (float32, in place) += delta (+ ``row``, one float32 vector [width] for every token); returns the
+        normed rows."""
+        return self._norm(residual, delta, None, weight, eps, unit_offset, out_dtype, residual.shape[0], row=row)
 
     def gather_add_rmsnorm(self, residual, delta, rows, weight, eps, unit_offset, out_dtype):
         return self._norm(residual, delta, rows, weight, eps, unit_offset, out_dtype, rows.numel())
@@ -1070,6 +1078,13 @@ class HipOps:
         p = [float(c) for c in consts] + [0.0, 0.0]
         return code, p[0], p[1]
 
+    @classmethod
+    def plain_kind(cls, activation) -> int:
+        """The code of a plain (ungated) activation: "silu", "gelu_tanh", "relu2" (the square of relu)."""
+        if activation not in cls.ACTIVATION_KINDS:
+            raise KernelError(f"activation {activation!r} is not offered (offered: {sorted(cls.ACTIVATION_KINDS)})")
+        return cls.ACTIVATION_KINDS[activation]
+
     def gated_act(self, gu, activation, out_dtype: Optional[torch.dtype] = None, group: int = 0) -> torch.Tensor:
         """act(gate) * up (or another gated pair, see ``gated_kind``) for gate/up columns [gate | up]
         (group 0) or alternating in groups of ``group`` columns (see ``pack_gate_up``)."""
@@ -1149,11 +1164,16 @@ class HipOps:
 
     def qkv_prepare(self, qkv, n_heads, n_kv, head_dim, value_dim, positions, act_dtype, q_norm=None, k_norm=None,
                     qk_eps: float = 0.0, rotation=None, value_norm_eps=None, value_rotation=None,
-                    k_cache=None, v_cache=None, slots=None, page_size: int = 0) -> torch.Tensor:
+                    k_cache=None, v_cache=None, slots=None, page_size: int = 0, bias=None, row_scales=None,
+                    norm_over_projection: bool = False, values_from_keys: bool = False) -> torch.Tensor:
         """From a projection's rows [q | k | v | ...] (a tensor or a ``SplitSum``): normed (weights
         ``q_norm`` / ``k_norm`` of head_dim elements, or none) and rotated queries [N, n_heads * head_dim];
         normed, rotated keys and unit-normed (``value_norm_eps``), rotated (``value_rotation``) values
-        into the pages (``n_kv`` 0: queries only)."""
+        into the pages (``n_kv`` 0: queries only).  ``bias`` (float32, one number per column of the projection)
+        is added first.  ``values_from_keys``: the rows are [q | k | ...] and a token's values are its keys as
+        projected (biased, before the norm).  ``norm_over_projection``: the weights are as wide as the q (k)
+        projection and no root mean square is taken here: it comes with ``row_scales`` (float32 [N, 2], from
+        ``qk_row_scales``), which multiply a token's queries (column 0) and keys (column 1) after the weights."""
         n_splits, round_sum, src = 1, 0, qkv
         if isinstance(qkv, SplitSum):
             qkv.check_live()
@@ -1164,8 +1184,16 @@ class HipOps:
             self._rows(qkv, "qkv")
             n, cols = qkv.shape
             stride = qkv.stride(0)
-        if cols < n_heads * head_dim + n_kv * (head_dim + value_dim):
+        if cols < n_heads * head_dim + n_kv * (head_dim + (0 if values_from_keys else value_dim)):
             raise KernelError(f"qkv rows have {cols} elements, fewer than the heads need")
+        if values_from_keys and value_dim != head_dim:
+            raise KernelError("qkv_prepare: values that are the keys are as wide as the keys")
+        if bias is not None and (bias.dtype != torch.float32 or bias.numel() < cols or not bias.is_contiguous()):
+            raise KernelError("qkv_prepare: the bias is contiguous float32 with a number per column of the projection")
+        if row_scales is not None and (row_scales.dtype != torch.float32 or tuple(row_scales.shape) != (n, 2) or not row_scales.is_contiguous()):
+            raise KernelError("qkv_prepare: the rows' scales are contiguous float32 [N, 2]")
+        if norm_over_projection and (row_scales is None or q_norm is None or (n_kv > 0 and k_norm is None)):
+            raise KernelError("qkv_prepare: a norm over the whole projection takes its weights and the rows' scales")
         if positions.numel() != n or (n_kv > 0 and slots.numel() != n):
             raise KernelError("positions/slots do not match the number of tokens")
         q_out = torch.empty((n, n_heads * head_dim), dtype=act_dtype, device=src.device)
@@ -1179,10 +1207,11 @@ class HipOps:
         norm_w = q_norm if q_norm is not None else k_norm
         if q_norm is not None and k_norm is not None and q_norm.dtype != k_norm.dtype:
             raise KernelError("query and key norm weights differ in dtype")
-        for w in (q_norm, k_norm):
-            if w is not None and (w.numel() != head_dim or not w.is_contiguous()):
-                raise KernelError(f"a head norm's weight has {w.numel()} elements, heads have {head_dim}")
-        qk_norm = int(q_norm is not None or k_norm is not None)
+        for w, heads in ((q_norm, n_heads), (k_norm, n_kv)):
+            want = heads * head_dim if norm_over_projection else head_dim
+            if w is not None and not (norm_over_projection and heads == 0) and (w.numel() != want or not w.is_contiguous()):
+                raise KernelError(f"a norm's weight has {w.numel()} elements, {want} are normed together")
+        qk_norm = int(q_norm is not None or k_norm is not None) * (2 if norm_over_projection else 1)
         if qk_norm and (q_norm is None or k_norm is None):
             raise KernelError("queries and keys are normed together or not at all")
         for r in (rotation, value_rotation):
@@ -1204,10 +1233,36 @@ class HipOps:
                 int(bool(value_rotation is not None and value_rotation.interleaved)),
                 0 if value_rotation is None else value_rotation.cos.shape[0],
                 _ptr(k_cache) if n_kv else None, _ptr(v_cache) if n_kv else None, _ptr(slots) if n_kv else None,
-                int(page_size), int(tiled), self._stream(),
+                int(page_size), int(tiled), _ptr(bias), _ptr(row_scales), int(bool(values_from_keys)), self._stream(),
             )
         )
         return q_out
+
+    def qk_row_scales(self, proj, n_q_cols: int, n_k_cols: int, positions, bias=None, eps=None, temperature=None) -> torch.Tensor:
+        """float32 [N, 2]: what a token's queries (column 0) and keys (column 1) are multiplied with as wholes.  With
+        ``eps``: 1 / sqrt(mean(x^2) + eps) over the first ``n_q_cols`` columns of the projection (a tensor or a
+        ``SplitSum``) plus ``bias``, and over the next ``n_k_cols``.  With ``temperature`` = (coef, every): the queries'
+        factor 1 + coef ln(floor((p + 1) / every) + 1) at position p on top."""
+        n_splits, round_sum, src = 1, 0, proj
+        if isinstance(proj, SplitSum):
+            proj.check_live()
+            n_splits, round_sum, src = proj.n_splits, proj.round_sum, proj.tensor
+            n, cols = proj.shape
+            stride = cols
+        else:
+            self._rows(proj, "projection")
+            n, cols = proj.shape
+            stride = proj.stride(0)
+        if cols < n_q_cols + n_k_cols or positions.numel() != n or positions.dtype != torch.int32:
+            raise KernelError("qk_row_scales: the projection holds the query and key columns, and every token has an int32 position")
+        if bias is not None and (bias.dtype != torch.float32 or bias.numel() < n_q_cols + n_k_cols or not bias.is_contiguous()):
+            raise KernelError("qk_row_scales: the bias is contiguous float32 with a number per column")
+        coef, every = (0.0, 0) if temperature is None else (float(temperature[0]), int(temperature[1]))
+        out = torch.empty((n, 2), dtype=torch.float32, device=src.device)
+        self._check(self.lib.yk_qk_row_scales(src.data_ptr(), _code(src.dtype), n_splits, round_sum, stride, n, int(n_q_cols), int(n_k_cols),
+                                              _ptr(bias), int(eps is not None), float(eps or 0.0), positions.data_ptr(), coef, every,
+                                              out.data_ptr(), self._stream()))
+        return out
 
     @staticmethod
     def _gate_source(gate, n: int):
@@ -1221,15 +1276,18 @@ class HipOps:
 
     def attention_masked(self, q, n_heads, n_kv, head_dim, value_dim, k_cache, v_cache, page_size, scale, ctx, group,
                          window: int = 0, keep_first: int = 0, softcap: float = 0.0, value_rotation=None,
-                         gate=None, gate_col: int = 0, gate_elems: int = 1, distance_bias=None) -> torch.Tensor:
+                         gate=None, gate_col: int = 0, gate_elems: int = 1, distance_bias=None, sink=None) -> torch.Tensor:
         """softmax over the keys j <= p with (p - j < window or j < keep_first) of q . k * scale
         (squashed by ``softcap`` * tanh(s / ``softcap``) when set), times the values [N, n_heads *
         value_dim]; then, with ``value_rotation``, every head's output turned back by its token's
         position, and, with ``gate`` (the projection, a tensor or ``SplitSum``, whose columns
         ``gate_col`` + h hold the heads' gates), multiplied by the sigmoid of its gate (``gate_elems`` = value_dim:
         a gate per output element, in the columns ``gate_col`` + h * value_dim + d).  ``distance_bias`` (float32
-        [distances, n_heads]): row min(p - j, distances - 1) is added to the scaled scores of head h."""
+        [distances, n_heads]): row min(p - j, distances - 1) is added to the scaled scores of head h.  ``sink`` (float32
+        [n_heads]): exp(sink[h]) joins head h's denominator once; it has no key and no value."""
         self._rows(q, "queries")
+        if sink is not None and (sink.dtype != torch.float32 or sink.numel() != n_heads or not sink.is_contiguous()):
+            raise KernelError("attention_masked: the sinks are contiguous float32 [heads]")
         if distance_bias is not None and (distance_bias.dtype != torch.float32 or distance_bias.dim() != 2 or not distance_bias.is_contiguous()
                                           or distance_bias.shape[1] != n_heads or distance_bias.shape[0] < 1):
             raise KernelError("attention_masked: the distance bias is contiguous float32 [distances, heads]")
@@ -1251,7 +1309,7 @@ class HipOps:
                 None if vr is None else vr.cos.data_ptr(), None if vr is None else vr.sin.data_ptr(),
                 int(bool(vr is not None and vr.interleaved)), 0 if vr is None else vr.cos.shape[0],
                 _ptr(gsrc), 0 if gsrc is None else _code(gsrc.dtype), gsplits, ground, gstride, int(gate_col), int(gate_elems),
-                _ptr(distance_bias), 0 if distance_bias is None else distance_bias.shape[0], self._stream(),
+                _ptr(distance_bias), 0 if distance_bias is None else distance_bias.shape[0], _ptr(sink), self._stream(),
             )
         )
         return out
@@ -1651,26 +1709,30 @@ class HipOps:
         return out
 
     # --------------------------------------------------------------- mixture of experts
-    def moe_experts(self, x, token_ids, table, w_gate_up, w_down, activation) -> torch.Tensor:
+    def moe_experts(self, x, token_ids, table, w_gate_up, w_down, activation, input_per_token: bool = False) -> torch.Tensor:
         """Every token through the experts its id names in ``table`` [vocab, top]: returns float32
         rows [N * top, hidden], row n * top + k the output of token n's k-th expert (uncombined).
         ``w_gate_up`` [experts, 2, ff, hidden] (gate rows, then up rows), ``w_down`` [experts, hidden, ff].
         ``token_ids`` None: ``table`` has a row per token of the step (a router's choice) and ``x`` a row per
-        (token, k) already, [N * top, hidden] (what ``moe_router_topk`` returns)."""
+        (token, k) already, [N * top, hidden] (what ``moe_router_topk`` returns), or, with ``input_per_token``, a row per
+        token that all its experts read.  ``w_gate_up`` [experts, 1, ff, hidden]: experts without a gate, down(act(up x))
+        with ``activation`` a plain one (``plain_kind``)."""
         self._rows(x, "expert input")
         vocab, top = table.shape
         if token_ids is None:
-            n, hidden, x_top = vocab, x.shape[1], 1  # x_top: how many pairs share a row of x
-            if x.shape[0] != n * top:
-                raise KernelError("moe: with a choice per token the input has a row per (token, choice)")
+            n, hidden = vocab, x.shape[1]
+            x_top = top if input_per_token else 1  # x_top: how many pairs share a row of x
+            if x.shape[0] != (n if input_per_token else n * top):
+                raise KernelError("moe: with a choice per token the input has a row per (token, choice), or a row per token")
         else:
             (n, hidden), x_top = x.shape, top
         experts, two, ff, hid = w_gate_up.shape
-        if two != 2 or hid != hidden or tuple(w_down.shape) != (experts, hidden, ff) or not w_gate_up.is_contiguous() or not w_down.is_contiguous():
-            raise KernelError("moe: expert weights must be contiguous [experts, 2, ff, hidden] and [experts, hidden, ff]")
+        gated = two == 2
+        if two not in (1, 2) or hid != hidden or tuple(w_down.shape) != (experts, hidden, ff) or not w_gate_up.is_contiguous() or not w_down.is_contiguous():
+            raise KernelError("moe: expert weights must be contiguous [experts, 2 (or 1: no gate), ff, hidden] and [experts, hidden, ff]")
         if table.dtype != torch.int32 or not table.is_contiguous() or (token_ids is not None and (token_ids.dtype != torch.int32 or token_ids.numel() != n)):
             raise KernelError("moe: the table and the token ids are int32, one id per row")
-        kind, p0, p1 = self.gated_kind(activation)
+        kind, p0, p1 = self.gated_kind(activation) if gated else (self.plain_kind(activation), 0.0, 0.0)
         pairs = n * top
         dev = x.device
         rows = torch.empty((pairs, hidden), dtype=torch.float32, device=dev)
@@ -1691,14 +1753,14 @@ class HipOps:
                 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0):
             # many pairs an expert: both products as tiles of 128 x 128 through LDS (the grouped form of
             # ``gemm_tile``), the gated pair by the activation kernel between them
-            gu = torch.empty((pairs, 2 * ff), dtype=bf, device=dev)
+            gu = torch.empty((pairs, two * ff), dtype=bf, device=dev)
             self._check(
                 self.lib.yk_gemm_tile_grouped(
-                    x.data_ptr(), x.stride(0), order.data_ptr(), x_top, w_gate_up.data_ptr(), 2 * ff * hidden, hidden, gu.data_ptr(),
-                    _BF16, 2 * ff, None, tiles.data_ptr(), n_tiles.data_ptr(), max_tiles, 2 * ff, hidden, self._stream(),
+                    x.data_ptr(), x.stride(0), order.data_ptr(), x_top, w_gate_up.data_ptr(), two * ff * hidden, hidden, gu.data_ptr(),
+                    _BF16, two * ff, None, tiles.data_ptr(), n_tiles.data_ptr(), max_tiles, two * ff, hidden, self._stream(),
                 )
             )
-            y = self.gated_act(gu, activation, bf)
+            y = self.gated_act(gu, activation, bf) if gated else self.activation(gu, activation, bf)
             self._check(
                 self.lib.yk_gemm_tile_grouped(
                     y.data_ptr(), ff, None, 1, w_down.data_ptr(), hidden * ff, ff, rows.data_ptr(), _F32, hidden,
@@ -1711,7 +1773,7 @@ class HipOps:
             self.lib.yk_moe_gate_up(
                 x.data_ptr(), x.stride(0), _code(x.dtype), w_gate_up.data_ptr(), _code(w_gate_up.dtype), order.data_ptr(),
                 slot_expert.data_ptr(), tiles.data_ptr(), n_tiles.data_ptr(), tile_rows, max_tiles, pairs, x_top, hidden, ff,
-                kind, p0, p1, y.data_ptr(), self._stream(),
+                kind, p0, p1, y.data_ptr(), int(gated), self._stream(),
             )
         )
         self._check(
@@ -1722,26 +1784,45 @@ class HipOps:
         )
         return rows
 
-    def moe_router_topk(self, logits, x, top: int, experts: Optional[int] = None):
+    def moe_router_topk(self, logits, x, top: int, experts: Optional[int] = None, bias=None, scores: str = "sigmoid"):
         """From a router's float32 ``logits`` [N, >= experts] (``experts``: how many of a row's columns are experts; the
         rest is padding): the ``top`` experts with the largest logits of every token
         (int32 [N, top]; among equals the lower number) and the token's row of ``x`` once per chosen expert times the
-        expert's score sigmoid(logit) ([N * top, hidden] in x's dtype): the score weighs the expert's input."""
-        self._rows(x, "router input")
+        expert's score sigmoid(logit) ([N * top, hidden] in x's dtype): the score weighs the expert's input.  ``bias``
+        (float32 [experts]) joins the logits before the choice.  ``scores`` "softmax_of_chosen": nothing is copied (``x``
+        may be None); the second result is float32 [N, top], the softmax over the chosen logits alone, which weighs the
+        experts' outputs."""
         self._rows(logits, "router logits")
         n = logits.shape[0]
         experts = logits.shape[1] if experts is None else int(experts)
-        if logits.dtype != torch.float32 or experts > logits.shape[1] or x.shape[0] != n or not 1 <= top <= min(experts, 64):
+        if logits.dtype != torch.float32 or experts > logits.shape[1] or not 1 <= top <= min(experts, 64):
             raise KernelError("moe_router_topk: logits are float32 [N, >= experts], top between 1 and min(experts, 64)")
-        choice = torch.empty((n, top), dtype=torch.int32, device=x.device)
+        if bias is not None and (bias.dtype != torch.float32 or bias.numel() != experts or not bias.is_contiguous()):
+            raise KernelError("moe_router_topk: the bias is contiguous float32 [experts]")
+        choice = torch.empty((n, top), dtype=torch.int32, device=logits.device)
+        if scores == "softmax_of_chosen":
+            weights = torch.empty((n, top), dtype=torch.float32, device=logits.device)
+            self._check(self.lib.yk_moe_router_topk(logits.data_ptr(), logits.stride(0), experts, int(top), None, 0, _F32, 0, choice.data_ptr(),
+                                                    None, n, _ptr(bias), weights.data_ptr(), self._stream()))
+            return choice, weights
+        if scores != "sigmoid":
+            raise KernelError(f"moe_router_topk: scores {scores!r} are not offered")
+        self._rows(x, "router input")
+        if x.shape[0] != n:
+            raise KernelError("moe_router_topk: a row of x per row of logits")
         xs = torch.empty((n * top, x.shape[1]), dtype=x.dtype, device=x.device)
         self._check(self.lib.yk_moe_router_topk(logits.data_ptr(), logits.stride(0), experts, int(top), x.data_ptr(), x.stride(0), _code(x.dtype),
-                                                x.shape[1], choice.data_ptr(), xs.data_ptr(), n, self._stream()))
+                                                x.shape[1], choice.data_ptr(), xs.data_ptr(), n, _ptr(bias), None, self._stream()))
         return choice, xs
 
-    def moe_combine(self, dense, rows, top: int, weight: float = 1.0) -> torch.Tensor:
+    def moe_combine(self, dense, rows, top: int, weight: float = 1.0, row_weights=None) -> torch.Tensor:
         """float32 [N, width]: ``dense`` (a tensor, a ``SplitSum`` or None) + weight * the sum of each token's ``top``
-        consecutive rows of ``rows`` (float32 [N * top, width])."""
+        consecutive rows of ``rows`` (float32 [N * top, width]), each first multiplied by its entry of ``row_weights``
+        (float32 [N, top]) where given."""
+        if isinstance(dense, SplitAttention):
+            dense = dense.merge()
+        if row_weights is not None and (row_weights.dtype != torch.float32 or row_weights.numel() != rows.shape[0] or not row_weights.is_contiguous()):
+            raise KernelError("moe_combine: the rows' weights are contiguous float32, one per row")
         if rows.dtype != torch.float32 or not rows.is_contiguous() or rows.dim() != 2 or rows.shape[0] % top:
             raise KernelError("moe_combine: the experts' rows are contiguous float32 [N * top, width]")
         n, width = rows.shape[0] // top, rows.shape[1]
@@ -1753,7 +1834,7 @@ class HipOps:
             raise KernelError(f"moe_combine: the dense part {tuple(dense.shape)} does not match the rows {(n, width)}")
         out = torch.empty((n, width), dtype=torch.float32, device=rows.device)
         self._check(self.lib.yk_moe_combine(_ptr(src), 0 if src is None else _code(src.dtype), n_splits, round_sum, rows.data_ptr(),
-                                            int(top), float(weight), out.data_ptr(), n, width, self._stream()))
+                                            int(top), float(weight), out.data_ptr(), n, width, _ptr(row_weights), self._stream()))
         return out
 
     # ------------------------------------------------------------------- sampling
