@@ -132,7 +132,9 @@ extern "C" int yk_attn_generic(const void* q, int q_stride, void* out, const voi
 // plain ones are compiled without): the first `keep_first` keys of a request stay visible below
 // the window, a score s (times the scale) is squashed to cap * tanh(s / cap), and a learned bias per head
 // and distance (a float32 table [distances][heads], the last row for everything farther) is added to
-// the scaled, squashed score.
+// the scaled, squashed score; a sink per head (float32 [heads]) joins the softmax's denominator once as exp(sink):
+// where a column's keys are whole in one workgroup, when its sum of weights is inverted; where they were split,
+// in the merge of the splits (a split never adds it itself).
 //
 // Kept first keys add blocks of 64 keys in front of the window's: a kernel numbers the blocks it
 // walks "virtually", the window's blocks by their own number and the n_first blocks of kept keys
@@ -258,7 +260,7 @@ __global__ __launch_bounds__(64 * W, 2) void attn_mfma_kernel(
     int page_size, int n_heads, int n_kv, int hpt, int chunks, float scale_log2, int window,
     int n_splits, float* __restrict__ ws_o, float* __restrict__ ws_ml, RopeSrc rs, int keep_first_arg = 0,
     float cap_over_scale = 0.f, float scale_over_cap_2log2e = 0.f, const float* __restrict__ dist_bias = nullptr,
-    int bias_rows = 0, float inv_scale = 0.f) {
+    int bias_rows = 0, float inv_scale = 0.f, const float* __restrict__ sink = nullptr) {
   const int keep_first = EXT ? keep_first_arg : 0;
   constexpr int KS = D / 32;  // matrix-core steps over the head dimension
   constexpr int DT = D / 16;  // output tiles over the head dimension
@@ -673,6 +675,8 @@ __global__ __launch_bounds__(64 * W, 2) void attn_mfma_kernel(
 
   if (n_splits == 1) {
     if (col_ok) {
+      // (m and l are in powers of two: the sink's share is 2^(sink log2(e) - m))
+      if (EXT && sink != nullptr) l += fast_exp2(fmaf(sink[h_base + hh], 1.4426950408889634f, -m));
       const float inv = 1.f / l;
       bf16_t* op = out + (static_cast<size_t>(tok0 + tt) * n_heads + h_base + hh) * D + 4 * gq;
 #pragma unroll
@@ -716,7 +720,8 @@ __global__ __launch_bounds__(256, CT == 1 ? 3 : 2) void attn_mfma_prefill_kernel
     const int32_t* __restrict__ tiles, const int32_t* __restrict__ block_table, int table_width,
     int page_size, int n_heads, int n_kv, int hpt, int chunks, float scale_log2, int window,
     int n_splits, float* __restrict__ ws_o, float* __restrict__ ws_ml, int pages_lds_limit, int keep_first_arg,
-    float cap_over_scale, float scale_over_cap_2log2e, const float* __restrict__ dist_bias, int bias_rows, float inv_scale) {
+    float cap_over_scale, float scale_over_cap_2log2e, const float* __restrict__ dist_bias, int bias_rows, float inv_scale,
+    const float* __restrict__ sink) {
   constexpr int KS = D / 32, DT = D / 16;
   const int keep_first = EXT ? keep_first_arg : 0;
   constexpr int KROW = D + 8;   // bf16 elements per parked key row
@@ -1026,6 +1031,7 @@ __global__ __launch_bounds__(256, CT == 1 ? 3 : 2) void attn_mfma_prefill_kernel
       continue;
     }
     if (col_ok[c]) {
+      if (EXT && sink != nullptr) lc += fast_exp2(fmaf(sink[h_base + hh], 1.4426950408889634f, -m[c]));
       const float inv = 1.f / lc;
       bf16_t* op = out + (static_cast<size_t>(tile_tok0 + tok_c[c]) * n_heads + h_base + hh) * D + 4 * gq;
 #pragma unroll
@@ -1046,7 +1052,8 @@ __global__ __launch_bounds__(256, CT == 1 ? 3 : 2) void attn_mfma_prefill_kernel
 template <int D>
 __global__ __launch_bounds__(256) void attn_combine_kernel(
     bf16_t* __restrict__ out, const int32_t* __restrict__ tiles, int n_heads, int n_kv, int hpt,
-    int chunks, int n_splits, const float* __restrict__ ws_o, const float* __restrict__ ws_ml, int parts) {
+    int chunks, int n_splits, const float* __restrict__ ws_o, const float* __restrict__ ws_ml, int parts,
+    const float* __restrict__ sink) {
   const int t = blockIdx.x / parts, part = blockIdx.x % parts;
   const int tpt_ = 16 / hpt;
   const int tok0 = tiles[4 * t + 1] + part * tpt_, ntok = tiles[4 * t + 2] - part * tpt_;
@@ -1062,7 +1069,8 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(
     // columns left over stand for nothing, not for the next part's first token)
     if (tt >= min(ntok, tpt_) || hh >= heads_here) continue;
     float merged[4];
-    attn_merge_splits(ws_o, ws_ml, w0 * 16 + c, n_splits, D, d, merged);
+    attn_merge_splits(ws_o, ws_ml, w0 * 16 + c, n_splits, D, d, merged,
+                      sink != nullptr ? sink[h_base + hh] * 1.4426950408889634f : -INFINITY);
     u32x2_t o;
     o[0] = pack_bf16x2(merged[0], merged[1]);
     o[1] = pack_bf16x2(merged[2], merged[3]);
@@ -1102,7 +1110,7 @@ extern "C" int yk_attn_mfma_prefill(const void* q, int q_stride, void* out, cons
                                     int head_dim, int n_heads, int n_kv, float scale, int window,
                                     int n_splits, int col_tiles, float* workspace, size_t workspace_floats,
                                     int pages_lds_limit, int keep_first, float softcap, const float* dist_bias, int bias_rows,
-                                    hipStream_t stream) {
+                                    const float* sink, hipStream_t stream) {
   YK_REQUIRE(n_tiles >= 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0, "attn_mfma_prefill: bad head counts");
   YK_REQUIRE(col_tiles == 1 || col_tiles == 2, "attn_mfma_prefill: a wave has 1 or 2 column tiles");
   YK_REQUIRE(yk_attn_mfma_supported(head_dim), "attn_mfma_prefill: head_dim must be 64 or 128");
@@ -1116,7 +1124,7 @@ extern "C" int yk_attn_mfma_prefill(const void* q, int q_stride, void* out, cons
   YK_REQUIRE(keep_first >= 0 && softcap >= 0.f, "attn_mfma_prefill: keep_first and softcap must not be negative");
   YK_REQUIRE(dist_bias == nullptr || bias_rows >= 1, "attn_mfma_prefill: an empty table of biases");
   if (n_tiles == 0) return 0;
-  const bool ext = (keep_first > 0 && window > 0) || softcap > 0.f || dist_bias != nullptr;
+  const bool ext = (keep_first > 0 && window > 0) || softcap > 0.f || dist_bias != nullptr || sink != nullptr;
   const float inv_scale = 1.f / scale;
   const float cap_over_scale = softcap > 0.f ? softcap / scale : 0.f;
   const float scale_over_cap = softcap > 0.f ? scale / softcap * 2.f * 1.4426950408889634f : 0.f;
@@ -1134,7 +1142,7 @@ extern "C" int yk_attn_mfma_prefill(const void* q, int q_stride, void* out, cons
   static_cast<const bf16_t*>(q), q_stride, static_cast<bf16_t*>(out), static_cast<const bf16_t*>(k_cache),     \
       static_cast<const bf16_t*>(v_cache), tiles, block_table, table_width, page_size, n_heads, n_kv, hpt,     \
       chunks, scale_log2, window, n_splits, ws_o, ws_ml, pages_lds_limit, keep_first, cap_over_scale, scale_over_cap, \
-      dist_bias, bias_rows, inv_scale
+      dist_bias, bias_rows, inv_scale, sink
 #define YK_PF(DD, BIP)                                                                                       \
   if (ext && col_tiles == 2)                                                                                 \
     attn_mfma_prefill_kernel<DD, BIP, 2, true><<<grid, block, 0, stream>>>(YK_PF_ARGS);                      \
@@ -1156,9 +1164,9 @@ extern "C" int yk_attn_mfma_prefill(const void* q, int q_stride, void* out, cons
   if (n_splits > 1) {
     dim3 cgrid(4 * col_tiles * n_tiles, n_kv * chunks);
     if (head_dim == 64)
-      attn_combine_kernel<64><<<cgrid, 256, 0, stream>>>(static_cast<bf16_t*>(out), tiles, n_heads, n_kv, hpt, chunks, n_splits, ws_o, ws_ml, 4 * col_tiles);
+      attn_combine_kernel<64><<<cgrid, 256, 0, stream>>>(static_cast<bf16_t*>(out), tiles, n_heads, n_kv, hpt, chunks, n_splits, ws_o, ws_ml, 4 * col_tiles, sink);
     else
-      attn_combine_kernel<128><<<cgrid, 256, 0, stream>>>(static_cast<bf16_t*>(out), tiles, n_heads, n_kv, hpt, chunks, n_splits, ws_o, ws_ml, 4 * col_tiles);
+      attn_combine_kernel<128><<<cgrid, 256, 0, stream>>>(static_cast<bf16_t*>(out), tiles, n_heads, n_kv, hpt, chunks, n_splits, ws_o, ws_ml, 4 * col_tiles, sink);
     return yk_check_launch("attn_combine");
   }
   return 0;
@@ -1173,11 +1181,12 @@ static int launch_attn_mfma(const void* q, int q_stride, void* out, const void* 
                             int page_size, int head_dim, int n_heads, int n_kv, float scale, int window,
                             int n_waves, int n_splits, float* workspace, size_t workspace_floats,
                             int leave_splits, const RopeSrc* rope, bool rope_f32, hipStream_t stream, int keep_first = 0,
-                            float softcap = 0.f, const float* dist_bias = nullptr, int bias_rows = 0) {
+                            float softcap = 0.f, const float* dist_bias = nullptr, int bias_rows = 0, const float* sink = nullptr) {
   YK_REQUIRE(n_tiles >= 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0, "attn_mfma: bad head counts");
+  YK_REQUIRE(sink == nullptr || !leave_splits, "attn_mfma: splits that another kernel merges cannot carry a sink");
   YK_REQUIRE(keep_first >= 0 && softcap >= 0.f, "attn_mfma: keep_first and softcap must not be negative");
   YK_REQUIRE(dist_bias == nullptr || bias_rows >= 1, "attn_mfma: an empty table of biases");
-  const bool ext = (keep_first > 0 && window > 0) || softcap > 0.f || dist_bias != nullptr;
+  const bool ext = (keep_first > 0 && window > 0) || softcap > 0.f || dist_bias != nullptr || sink != nullptr;
   const float inv_scale = scale > 0.f ? 1.f / scale : 0.f;
   YK_REQUIRE(!(ext && rope), "attn_mfma: kept first keys and squashed scores are not offered with rotary inside the launch");
   const float cap_over_scale = softcap > 0.f ? softcap / scale : 0.f;
@@ -1218,11 +1227,11 @@ static int launch_attn_mfma(const void* q, int q_stride, void* out, const void* 
   }
 #define YK_LAUNCH_EXT(DD)                                                                          \
   if (tiled) {                                                                                     \
-    if (n_waves == 1) attn_mfma_kernel<DD, 1, true, 0, true><<<grid, block, 0, stream>>>(YK_ARGS, keep_first, cap_over_scale, scale_over_cap, dist_bias, bias_rows, inv_scale); \
-    else attn_mfma_kernel<DD, 4, true, 0, true><<<grid, block, 0, stream>>>(YK_ARGS, keep_first, cap_over_scale, scale_over_cap, dist_bias, bias_rows, inv_scale); \
+    if (n_waves == 1) attn_mfma_kernel<DD, 1, true, 0, true><<<grid, block, 0, stream>>>(YK_ARGS, keep_first, cap_over_scale, scale_over_cap, dist_bias, bias_rows, inv_scale, sink); \
+    else attn_mfma_kernel<DD, 4, true, 0, true><<<grid, block, 0, stream>>>(YK_ARGS, keep_first, cap_over_scale, scale_over_cap, dist_bias, bias_rows, inv_scale, sink); \
   } else {                                                                                         \
-    if (n_waves == 1) attn_mfma_kernel<DD, 1, false, 0, true><<<grid, block, 0, stream>>>(YK_ARGS, keep_first, cap_over_scale, scale_over_cap, dist_bias, bias_rows, inv_scale); \
-    else attn_mfma_kernel<DD, 4, false, 0, true><<<grid, block, 0, stream>>>(YK_ARGS, keep_first, cap_over_scale, scale_over_cap, dist_bias, bias_rows, inv_scale); \
+    if (n_waves == 1) attn_mfma_kernel<DD, 1, false, 0, true><<<grid, block, 0, stream>>>(YK_ARGS, keep_first, cap_over_scale, scale_over_cap, dist_bias, bias_rows, inv_scale, sink); \
+    else attn_mfma_kernel<DD, 4, false, 0, true><<<grid, block, 0, stream>>>(YK_ARGS, keep_first, cap_over_scale, scale_over_cap, dist_bias, bias_rows, inv_scale, sink); \
   }
 #define YK_LAUNCH(DD)                                                                              \
   if (ext) { YK_LAUNCH_EXT(DD) } else                                                              \
@@ -1230,7 +1239,7 @@ static int launch_attn_mfma(const void* q, int q_stride, void* out, const void* 
   if (yk_check_launch("attn_mfma")) return -1;                                                     \
   if (n_splits > 1 && !leave_splits) {                                                             \
     attn_combine_kernel<DD><<<dim3(n_tiles, n_kv * chunks), 256, 0, stream>>>(                     \
-        static_cast<bf16_t*>(out), tiles, n_heads, n_kv, hpt, chunks, n_splits, ws_o, ws_ml, 1);   \
+        static_cast<bf16_t*>(out), tiles, n_heads, n_kv, hpt, chunks, n_splits, ws_o, ws_ml, 1, sink); \
     if (yk_check_launch("attn_combine")) return -1;                                                \
   }
   if (head_dim == 64) {
@@ -1251,10 +1260,10 @@ extern "C" int yk_attn_mfma(const void* q, int q_stride, void* out, const void* 
                             int head_dim, int n_heads, int n_kv, float scale, int window,
                             int n_waves, int n_splits, float* workspace, size_t workspace_floats,
                             int leave_splits, int keep_first, float softcap, const float* dist_bias, int bias_rows,
-                            hipStream_t stream) {
+                            const float* sink, hipStream_t stream) {
   return launch_attn_mfma(q, q_stride, out, k_cache, v_cache, tiles, n_tiles, block_table, table_width, page_size,
                           head_dim, n_heads, n_kv, scale, window, n_waves, n_splits, workspace, workspace_floats,
-                          leave_splits, nullptr, false, stream, keep_first, softcap, dist_bias, bias_rows);
+                          leave_splits, nullptr, false, stream, keep_first, softcap, dist_bias, bias_rows, sink);
 }
 
 // yk_attn_mfma for a step of single tokens (every tile holds ONE token), with rotary + append
@@ -1314,8 +1323,8 @@ extern "C" int yk_attn_combine(void* out, const int32_t* tiles, int n_tiles, int
   const float* ws_ml = workspace + (need / (head_dim + 2)) * head_dim;
   const dim3 grid(n_tiles, n_kv * chunks);
   if (head_dim == 64)
-    attn_combine_kernel<64><<<grid, 256, 0, stream>>>(static_cast<bf16_t*>(out), tiles, n_heads, n_kv, hpt, chunks, n_splits, ws_o, ws_ml, 1);
+    attn_combine_kernel<64><<<grid, 256, 0, stream>>>(static_cast<bf16_t*>(out), tiles, n_heads, n_kv, hpt, chunks, n_splits, ws_o, ws_ml, 1, nullptr);
   else
-    attn_combine_kernel<128><<<grid, 256, 0, stream>>>(static_cast<bf16_t*>(out), tiles, n_heads, n_kv, hpt, chunks, n_splits, ws_o, ws_ml, 1);
+    attn_combine_kernel<128><<<grid, 256, 0, stream>>>(static_cast<bf16_t*>(out), tiles, n_heads, n_kv, hpt, chunks, n_splits, ws_o, ws_ml, 1, nullptr);
   return yk_check_launch("attn_combine");
 }

@@ -185,12 +185,13 @@ __host__ __device__ inline int attn_heads_per_tile(int n_heads, int n_kv) {
 // groups numbered (tile * groups_y + kv head * chunks + chunk) * n_splits + split.
 // Four consecutive output elements of one column, merged over its splits: weights
 // exp2(m_s - max m), in the order of s.  `col0` is the column's index in split 0
-// (group * 16 + column); split s lies 16 columns further each.
+// (group * 16 + column); split s lies 16 columns further each.  `sink_log2` (-inf: none): a term 2^sink_log2 that joins
+// the sum of weights once, with no output of its own.
 __device__ __forceinline__ void attn_merge_splits(const float* __restrict__ o, const float* __restrict__ ml,
                                                   size_t col0, int n_splits, int head_dim, int d,
-                                                  float out[4]) {
+                                                  float out[4], float sink_log2 = -INFINITY) {
   const float* mlc = ml + col0 * 2;
-  float m_max = -INFINITY;
+  float m_max = sink_log2;
 #pragma unroll 4
   for (int s = 0; s < n_splits; ++s) m_max = fmaxf(m_max, mlc[static_cast<size_t>(s) * 32]);
   float num[4] = {0.f, 0.f, 0.f, 0.f};
@@ -205,6 +206,7 @@ __device__ __forceinline__ void attn_merge_splits(const float* __restrict__ o, c
     num[3] += w * v.w;
     den += w * mlc[static_cast<size_t>(s) * 32 + 1];
   }
+  if (sink_log2 != -INFINITY) den += exp2f(sink_log2 - m_max);
   const float inv = 1.f / den;
 #pragma unroll
   for (int e = 0; e < 4; ++e) out[e] = num[e] * inv;

@@ -180,11 +180,11 @@ _SIGNATURES = {
     "yk_attn_tokens_per_tile": ([_c_int, _c_int], _c_int),
     "yk_attn_mfma_workspace": ([_c_int, _c_int, _c_int, _c_int, _c_int], _c_size_t),
     "yk_attn_mfma_prefill": (
-        [_vp, _c_int, _vp, _vp, _vp, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_int, _vp, _c_size_t, _c_int, _c_int, _c_float, _vp, _c_int, _vp],
+        [_vp, _c_int, _vp, _vp, _vp, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_int, _vp, _c_size_t, _c_int, _c_int, _c_float, _vp, _c_int, _vp, _vp],
         _c_int,
     ),
     "yk_attn_mfma": (
-        [_vp, _c_int, _vp, _vp, _vp, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_int, _vp, _c_size_t, _c_int, _c_int, _c_float, _vp, _c_int, _vp],
+        [_vp, _c_int, _vp, _vp, _vp, _vp, _c_int, _vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_int, _vp, _c_size_t, _c_int, _c_int, _c_float, _vp, _c_int, _vp, _vp],
         _c_int,
     ),
     "yk_attn_mfma_rope": (
@@ -917,10 +917,15 @@ class HipOps:
         short spans can rotate queries and append keys and values itself."""
         return act_dtype == torch.bfloat16 and bool(self._ask("yk_attn_mfma_supported", head_dim))
 
+    def attention_takes_sink(self, act_dtype: torch.dtype, head_dim: int) -> bool:
+        """Whether ``attention`` takes ``sink=`` at these sizes (the matrix-core kernels do; elsewhere sinks are
+        ``attention_masked``'s)."""
+        return self.attention_can_rotate(act_dtype, head_dim)
+
     def attention(self, qkv, n_heads, n_kv, head_dim, k_cache, v_cache, page_size,
                   scale, window, ctx, group, tiles, long_tiles=None, plan=None, long_plan=None,
                   long_col_tiles: int = 1, token_cols=None, rope: Optional["RopeInLaunch"] = None,
-                  keep_first: int = 0, softcap: float = 0.0, distance_bias=None):
+                  keep_first: int = 0, softcap: float = 0.0, distance_bias=None, sink=None):
         """Queries are the first n_heads heads of each row of ``qkv`` (whatever follows
         them in the row is skipped); keys and values come from the cache through the
         block table of ``group``.  ``long_tiles`` hold up to
@@ -957,8 +962,10 @@ class HipOps:
             and qkv.stride(0) % 8 == 0
             and qkv.data_ptr() % 16 == 0
         )
-        if (keep_first or softcap or distance_bias is not None) and not use_mfma:
-            raise KernelError("attention: kept first keys, squashed scores and biases per distance outside the matrix-core kernels' sizes are attention_masked's")
+        if (keep_first or softcap or distance_bias is not None or sink is not None) and not use_mfma:
+            raise KernelError("attention: kept first keys, squashed scores, biases per distance and sinks outside the matrix-core kernels' sizes are attention_masked's")
+        if sink is not None and (sink.dtype != torch.float32 or sink.numel() != n_heads or not sink.is_contiguous()):
+            raise KernelError("attention: the sinks are contiguous float32 [heads]")
         if distance_bias is not None and (distance_bias.dtype != torch.float32 or distance_bias.dim() != 2 or not distance_bias.is_contiguous()
                                           or distance_bias.shape[1] != n_heads or distance_bias.shape[0] < 1):
             raise KernelError("attention: the distance bias is contiguous float32 [distances, heads]")
@@ -976,7 +983,7 @@ class HipOps:
                     long_tiles.data_ptr(), n_long, bt.data_ptr(), bt.shape[1], page_size, head_dim,
                     n_heads, n_kv, float(scale), int(window), long_splits, int(long_col_tiles), _ptr(ws),
                     0 if ws is None else ws.numel(), int(self.long_span_pages_in_lds), int(keep_first), float(softcap),
-                    _ptr(distance_bias), bias_rows, self._stream(),
+                    _ptr(distance_bias), bias_rows, _ptr(sink), self._stream(),
                 )
             )
         if use_mfma and tiles.shape[0] == 0:
@@ -989,13 +996,14 @@ class HipOps:
             waves, splits = plan or self.attention_plan(n_tiles * n_kv * chunks, key_blocks)
             ws_floats = self._ask("yk_attn_mfma_workspace", n_tiles, n_heads, n_kv, head_dim, splits)
             ws = self._ws(ws_floats) if ws_floats else None
-            leave = bool(token_cols is not None and splits > 1 and n <= MERGE_IN_PRODUCT_MAX_TOKENS and (long_tiles is None or long_tiles.shape[0] == 0))
+            leave = bool(token_cols is not None and splits > 1 and n <= MERGE_IN_PRODUCT_MAX_TOKENS and (long_tiles is None or long_tiles.shape[0] == 0)
+                         and sink is None)  # (a sink joins in the merge kernel)
             self._check(
                 self.lib.yk_attn_mfma(
                     qkv.data_ptr(), qkv.stride(0), out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
                     tiles.data_ptr(), n_tiles, bt.data_ptr(), bt.shape[1], page_size, head_dim, n_heads, n_kv,
                     float(scale), int(window), waves, splits, _ptr(ws), 0 if ws is None else ws.numel(), int(leave),
-                    int(keep_first), float(softcap), _ptr(distance_bias), bias_rows, self._stream(),
+                    int(keep_first), float(softcap), _ptr(distance_bias), bias_rows, _ptr(sink), self._stream(),
                 )
             )
             if leave:
