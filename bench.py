@@ -36,6 +36,10 @@ feed-forward weights.
 attention with a bias per distance, dense and routed feed-forwards) beside the Nutavik configuration of equal width,
 depth, heads, latent and feed-forward sizes (the closest of the engine's models: latent attention and matrix-state
 recurrences) and the Llama configuration of equal size.
+``--design bekedra`` measures the Bekedra design (two attention mixers in parallel blocks with routed experts without
+gates, a stretch of layers run twice) beside the Mesolix configuration of equal width, heads, experts and depth (the
+closest of the engine's models: the same attention and grouped-expert kernels) and the Llama configuration of equal
+size.
 """
 import argparse
 import json
@@ -412,7 +416,7 @@ def _op_costs(ops, hb):
     def moe(a, kw, out):
         x, table, wgu, wd = a[0], a[2], a[3], a[4]
         m, top, experts = x.shape[0], table.shape[1], wgu.shape[0]
-        if a[1] is None:  # a router's choice: the input has a row per (token, chosen expert) already
+        if a[1] is None and not kw.get("input_per_token"):  # a router's choice: the input has a row per (token, chosen expert) already
             m //= top
         per_expert = wgu[0].numel() + wd[0].numel()
         return 2.0 * m * top * per_expert, 2.0 * min(m * top, experts) * per_expert + nbytes(x) * (1 + top) + 4.0 * m * top * x.shape[1]
@@ -456,7 +460,7 @@ def _op_costs(ops, hb):
             "rope_append": moved, "causal_conv": moved, "gated_act": moved, "round_rows": moved, "embed": moved,
             "sandwich_norm": moved, "activation": moved, "latent_prepare": moved, "head_linear": head_linear,
             "latent_attention": latent_attention, "linear_state_scan": state_scan, "gated_head_norm": moved, "conv_state_push": moved, "moe_router_topk": moved,
-            "moe_combine": moved, "attention_finish": moved}
+            "moe_combine": moved, "attention_finish": moved, "qk_row_scales": moved}
 
 
 def per_op_times(runner, vocab: int, gen, batch: int, prompt_len: int, prefill_len: int):
@@ -546,9 +550,10 @@ def design_compare(args) -> int:
     the Llama configuration of equal size; one JSON line a size."""
     import torch
 
-    from yalis_amd.models.presets import llama_like, nutavik_like
+    from yalis_amd.models.presets import layer_runs, llama_like, mesolix_like, nutavik_like
 
-    sizes = {"suranex": ("suranex-2k", "suranex-4k"), "nutavik": ("nutavik-2k", "nutavik-4k"), "mesolix": ("mesolix-2k", "mesolix-4k")}[args.design]
+    sizes = {"suranex": ("suranex-2k", "suranex-4k"), "nutavik": ("nutavik-2k", "nutavik-4k"), "mesolix": ("mesolix-2k", "mesolix-4k"),
+             "bekedra": ("bekedra-2k", "bekedra-4k")}[args.design]
     if args.design_shape:
         sizes = (args.design_shape,)
     for name in sizes:
@@ -558,6 +563,8 @@ def design_compare(args) -> int:
         beside = [("design", cfg)]
         if args.design == "mesolix":
             beside.append(("nutavik_of_equal_size", nutavik_like(cfg)))
+        if args.design == "bekedra":
+            beside.append(("mesolix_of_equal_size", mesolix_like(cfg)))
         beside.append(("llama_of_equal_size", llama_like(cfg)))
         for who, c in beside:
             gen = torch.Generator().manual_seed(0)
@@ -568,7 +575,7 @@ def design_compare(args) -> int:
             runner = engine.runner
             pf, _ = prefill_run(runner, vocab, gen, args.prefill_len, runs=4)
             dt, _ = decode_run(runner, vocab, gen, args.batch, args.prompt_len, steps, args.warmup)
-            entry = {"layers": len(c["layers"]) if "layers" in c else c["num_hidden_layers"],
+            entry = {"layers": layer_runs(c) if "layers" in c else c["num_hidden_layers"],
                      "prefill_tok_s": round(args.prefill_len / pf, 1), "prefill_ms": round(1e3 * pf, 3),
                      "decode_tok_s": round(args.batch * steps / dt, 1), "decode_ms_per_step": round(1e3 * dt / steps, 4)}
             entry["ops"] = per_op_times(runner, vocab, gen, args.batch, args.prompt_len, args.prefill_len)
@@ -581,9 +588,9 @@ def design_compare(args) -> int:
 
 def main() -> int:
     ap = argparse.ArgumentParser()
-    ap.add_argument("--design", choices=("suranex", "nutavik", "mesolix"), default=None,
+    ap.add_argument("--design", choices=("suranex", "nutavik", "mesolix", "bekedra"), default=None,
                     help="measure instead another design's prefill and decode at a few layer sizes, beside the Llama configuration of equal size, with the time and the bound of every kind of kernel")
-    ap.add_argument("--design-shape", default=None, help="with --design: one of its shapes only (suranex-2k, suranex-4k, nutavik-2k, nutavik-4k, mesolix-2k, mesolix-4k)")
+    ap.add_argument("--design-shape", default=None, help="with --design: one of its shapes only (suranex-2k, suranex-4k, nutavik-2k, nutavik-4k, mesolix-2k, mesolix-4k, bekedra-2k, bekedra-4k)")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=32)
     ap.add_argument("--warmup", type=int, default=4)

@@ -146,6 +146,27 @@ def test_long_prompt_in_one_step(backend, name):
     X.assert_matches(got, want, dtype == "bfloat16", f"{name}/long prompt in portions", gaps)
 
 
+@pytest.mark.parametrize("backend", BACKENDS)
+def test_a_width_whose_products_come_in_slices(backend):
+    """Width 1,024 with heads of 128: for few tokens the projections' products are left as slices that the next
+    kernel sums (the mixer's output waits in the library's workspace while nothing else may take it); single tokens
+    behind a prompt, and the prompt in portions."""
+    device, dtype = backend
+    if device == "cpu":
+        pytest.skip("the plain ops have no slices; the GPU runs it")
+    cfg = X.model(300, 1024, 1e-6, 32.0, [
+        (X.sinked(8, 2, 128, 128, 0.09, softcap=30.0, rot=(64, 10000.0, 8.0, 1.0, 4.0, 32)), X.moe(4, 2, 256)),
+        (X.tempered(8, 2, 128, 0.09, 0.3, 32), X.moe(4, 2, 256)),
+    ], loop=(0, 2, 2))
+    weights = X.random_weights(cfg, seed=51)
+    reqs = X.make_requests(cfg, [70, 9], seed=5)
+    want, gaps = X.plain_logits_and_gaps(cfg, weights, reqs)
+    for make in (lambda r: C.trace_tail(r, tail=20), C.trace_portions, C.trace_mixed):
+        runner = X.make_runner(cfg, weights, dtype, device, ops_for(device), 64, 4)
+        got, _ = C.run_trace(runner, make(reqs))
+        X.assert_matches(got, want, dtype == "bfloat16", "width 1,024", gaps)
+
+
 def _one_layer(layer, ff, width=32, eps=1e-5, scale=2.0, loop=None, vocab=80):
     return X.model(vocab, width, eps, scale, [(layer, ff)], loop=loop)
 

@@ -239,3 +239,45 @@ def test_command_line_generates_with_mesolix():
         cwd=ROOT, capture_output=True, text=True, timeout=600,
     )
     assert proc.returncode == 0, proc.stderr[-2000:]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+def test_trace_run_cli_with_bekedra(tmp_path, dtype):
+    """The same program with a Bekedra folder written by the random-weights mode: a mixed trace in a pool that
+    holds four requests (two kinds of attention in parallel blocks with routed experts, layers run twice with pages
+    of their own for every pass)."""
+    import bekedra_cases as B
+    from yalis_amd.models.presets import shape
+
+    cfg = shape("bekedra-tiny")[1]
+    folder = write_random_model(str(tmp_path / "m"), cfg, seed=6, dtype="bfloat16")
+    weights = {n: read_tensor(e).float() for n, e in index_folder(folder).items()}
+    reqs = B.make_requests(cfg, [70, 20, 130, 45, 64], seed=8)
+    steps = C.trace_mixed(reqs)
+    out = str(tmp_path / "out")
+    run_cli(folder, dtype, out, steps, 64 * C.pages_needed(steps, reqs, 64))
+    want, gaps = B.plain_logits_and_gaps(cfg, weights, reqs)
+    got, cached = {}, {}
+    for s in steps:
+        rows = np.fromfile(os.path.join(out, f"{s['step']}.f32"), dtype="<f4").reshape(-1, cfg["vocab"])
+        r = 0
+        for e in s["entries"]:
+            base = cached.get(e["id"], 0)
+            for w in e["want"]:
+                got.setdefault(e["id"], {})[base + w] = torch.from_numpy(rows[r].copy())
+                r += 1
+            cached[e["id"]] = base + len(e["tokens"])
+    B.assert_matches({k: torch.stack([d[i] for i in sorted(d)]) for k, d in got.items()}, want, dtype == "bfloat16", "trace_run", gaps)
+
+
+@pytest.mark.gpu
+def test_command_line_generates_with_bekedra():
+    """``python -m yalis_amd.infer --random bekedra-tiny``: the scheduler, the sampler and the decode graphs with a
+    model whose looped layers keep pages per pass."""
+    proc = subprocess.run(
+        [sys.executable, "-m", "yalis_amd.infer", "--random", "bekedra-tiny", "--random-prompts", "3,40", "--tokens-to-generate", "24",
+         "--max-batch-size", "3", "--max-length-of-generated-sequences", "128", "--temperature", "0.7", "--top-k", "20"],
+        cwd=ROOT, capture_output=True, text=True, timeout=600,
+    )
+    assert proc.returncode == 0, proc.stderr[-2000:]

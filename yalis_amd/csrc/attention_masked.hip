@@ -404,29 +404,57 @@ extern "C" int yk_qkv_prepare(const void* src, int src_dtype, int n_splits, int 
 // out[n][0] for the queries, out[n][1] for the keys: 1 / sqrt(mean(x^2) + eps) over all n_q_cols query columns (all
 // n_k_cols key columns) of the biased projection when `normed`, times, for the queries, the temperature
 // 1 + coef * ln(floor((p + 1) / every) + 1) of the token's position p when every > 0.  A workgroup a token.
-template <typename TS>
-__global__ __launch_bounds__(256) void qk_row_scales_kernel(
+template <typename TS, bool VEC>
+__global__ __launch_bounds__(1024) void qk_row_scales_kernel(
     const TS* __restrict__ src, int n_splits, size_t split_stride, int round_sum, int src_stride, int n_q_cols, int n_k_cols,
     const float* __restrict__ bias, int normed, float eps, const int32_t* __restrict__ positions, float temp_coef,
     int temp_every, float* __restrict__ out) {
-  __shared__ float scratch[17];
-  const int n = blockIdx.x;
+  __shared__ float part[16][2];
+  const int n = blockIdx.x, wave = threadIdx.x / 64, lane = threadIdx.x % 64, n_waves = blockDim.x / 64;
   float sq = 1.f, sk = 1.f;
   if (normed) {
     const TS* row = src + static_cast<size_t>(n) * src_stride;
+    const int total = n_q_cols + n_k_cols;
     float ssq = 0.f, ssk = 0.f;
-    for (int c = threadIdx.x; c < n_q_cols + n_k_cols; c += blockDim.x) {
-      float v = 0.f;
-      for (int s = 0; s < n_splits; ++s) v += to_f32<TS>(row[s * split_stride + c]);
-      v = as_output(v, round_sum);
-      if (bias != nullptr) v += bias[c];
-      if (c < n_q_cols) ssq = fmaf(v, v, ssq);
-      else ssk = fmaf(v, v, ssk);
+    if (VEC) {
+      // bfloat16 rows in pieces of 16 bytes (the launcher checked the alignment and that a piece holds queries or
+      // keys, never both)
+      for (int c = threadIdx.x * 8; c < total; c += 8 * blockDim.x) {
+        const uint4 raw = *reinterpret_cast<const uint4*>(reinterpret_cast<const bf16_t*>(row) + c);
+        float v[8] = {__uint_as_float(raw.x << 16), __uint_as_float(raw.x & 0xffff0000u), __uint_as_float(raw.y << 16),
+                      __uint_as_float(raw.y & 0xffff0000u), __uint_as_float(raw.z << 16), __uint_as_float(raw.z & 0xffff0000u),
+                      __uint_as_float(raw.w << 16), __uint_as_float(raw.w & 0xffff0000u)};
+        if (bias != nullptr) {
+          const float4 b0 = *reinterpret_cast<const float4*>(bias + c), b1 = *reinterpret_cast<const float4*>(bias + c + 4);
+          v[0] += b0.x, v[1] += b0.y, v[2] += b0.z, v[3] += b0.w, v[4] += b1.x, v[5] += b1.y, v[6] += b1.z, v[7] += b1.w;
+        }
+        float ss = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) ss = fmaf(v[e], v[e], ss);
+        if (c < n_q_cols) ssq += ss;
+        else ssk += ss;
+      }
+    } else {
+      for (int c = threadIdx.x; c < total; c += blockDim.x) {
+        float v = 0.f;
+#pragma unroll 8
+        for (int s = 0; s < n_splits; ++s) v += to_f32<TS>(row[s * split_stride + c]);
+        v = as_output(v, round_sum);
+        if (bias != nullptr) v += bias[c];
+        if (c < n_q_cols) ssq = fmaf(v, v, ssq);
+        else ssk = fmaf(v, v, ssk);
+      }
     }
-    ssq = block_sum(ssq, scratch);
-    ssk = block_sum(ssk, scratch);
-    sq = 1.f / sqrtf(ssq / static_cast<float>(n_q_cols) + eps);
-    if (n_k_cols > 0) sk = 1.f / sqrtf(ssk / static_cast<float>(n_k_cols) + eps);
+    ssq = wave_sum(ssq);
+    ssk = wave_sum(ssk);
+    if (lane == 0) part[wave][0] = ssq, part[wave][1] = ssk;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      ssq = ssk = 0.f;
+      for (int w = 0; w < n_waves; ++w) ssq += part[w][0], ssk += part[w][1];
+      sq = 1.f / sqrtf(ssq / static_cast<float>(n_q_cols) + eps);
+      if (n_k_cols > 0) sk = 1.f / sqrtf(ssk / static_cast<float>(n_k_cols) + eps);
+    }
   }
   if (threadIdx.x == 0) {
     if (temp_every > 0) sq *= 1.f + temp_coef * logf(static_cast<float>((positions[n] + 1) / temp_every + 1));
@@ -443,12 +471,22 @@ extern "C" int yk_qk_row_scales(const void* src, int src_dtype, int n_splits, in
   YK_REQUIRE(temp_every >= 0 && (temp_every == 0 || positions != nullptr) && eps >= 0.f, "qk_row_scales: bad constants");
   if (n_tokens == 0) return 0;
   const size_t stride = static_cast<size_t>(n_tokens) * src_stride;
+  // few tokens (single decoded ones, whose projection comes as slices): a token's columns over sixteen waves
+  const int grid = n_tokens, block = n_tokens <= 256 ? 1024 : 256;
+  const bool vec = src_dtype == YK_BF16 && n_splits == 1 && n_q_cols % 8 == 0 && n_k_cols % 8 == 0 && src_stride % 8 == 0 &&
+                   reinterpret_cast<uintptr_t>(src) % 16 == 0 && reinterpret_cast<uintptr_t>(bias) % 16 == 0;
   if (src_dtype == YK_F32)
-    qk_row_scales_kernel<float><<<n_tokens, 256, 0, stream>>>(static_cast<const float*>(src), n_splits, stride, round_sum, src_stride,
-                                                              n_q_cols, n_k_cols, bias, normed, eps, positions, temp_coef, temp_every, out);
+    qk_row_scales_kernel<float, false><<<grid, block, 0, stream>>>(static_cast<const float*>(src), n_splits, stride, round_sum, src_stride,
+                                                                 n_q_cols, n_k_cols, bias, normed, eps, positions, temp_coef,
+                                                                 temp_every, out);
+  else if (src_dtype == YK_BF16 && vec)
+    qk_row_scales_kernel<bf16_t, true><<<grid, block, 0, stream>>>(static_cast<const bf16_t*>(src), n_splits, stride, round_sum, src_stride,
+                                                                 n_q_cols, n_k_cols, bias, normed, eps, positions, temp_coef,
+                                                                 temp_every, out);
   else if (src_dtype == YK_BF16)
-    qk_row_scales_kernel<bf16_t><<<n_tokens, 256, 0, stream>>>(static_cast<const bf16_t*>(src), n_splits, stride, round_sum, src_stride,
-                                                               n_q_cols, n_k_cols, bias, normed, eps, positions, temp_coef, temp_every, out);
+    qk_row_scales_kernel<bf16_t, false><<<grid, block, 0, stream>>>(static_cast<const bf16_t*>(src), n_splits, stride, round_sum, src_stride,
+                                                                  n_q_cols, n_k_cols, bias, normed, eps, positions, temp_coef,
+                                                                  temp_every, out);
   else
     return yk_fail("qk_row_scales: unsupported dtype");
   return yk_check_launch("qk_row_scales");

@@ -103,12 +103,16 @@ template <typename T>
 __global__ __launch_bounds__(256) void moe_router_topk_kernel(const float* __restrict__ logits, int logits_stride, int n_experts, int top,
                                                               const T* __restrict__ x, int x_stride, int hidden,
                                                               int32_t* __restrict__ choice, T* __restrict__ xs,
-                                                              const float* __restrict__ bias, float* __restrict__ weights) {
-  extern __shared__ float sel[];  // [top] scores, then [top] numbers (as ints)
+                                                              const float* __restrict__ bias, float* __restrict__ weights, int n_tokens) {
+  extern __shared__ float sel_all[];  // per choosing wave: [top] scores, then [top] numbers (as ints)
+  // with weights every wave of the workgroup chooses for a token of its own (there is nothing to copy afterwards)
+  const bool per_wave = weights != nullptr;
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  float* sel = sel_all + (per_wave ? wave * 2 * top : 0);
   int* sel_e = reinterpret_cast<int*>(sel + top);
-  const int n = blockIdx.x, lane = threadIdx.x;
+  const int n = per_wave ? min(static_cast<int>(blockIdx.x) * 4 + wave, n_tokens - 1) : blockIdx.x;
   const float* row = logits + static_cast<size_t>(n) * logits_stride;
-  if (threadIdx.x < kWave) {
+  if (per_wave || threadIdx.x < kWave) {
     for (int k = 0; k < top; ++k) {
       float best = -INFINITY;
       int best_e = 0x7fffffff;
@@ -163,15 +167,15 @@ extern "C" int yk_moe_router_topk(const float* logits, int logits_stride, int n_
   YK_REQUIRE(weights != nullptr || (x != nullptr && hidden > 0 && x_stride >= hidden), "moe_router_topk: bad input rows");
   if (n_tokens == 0) return 0;
   const size_t lds = 2 * static_cast<size_t>(top) * sizeof(float);
-  if (weights != nullptr)  // one wave chooses and weighs; there is nothing to copy
-    moe_router_topk_kernel<float><<<n_tokens, 64, lds, stream>>>(logits, logits_stride, n_experts, top, nullptr, 0, 0, choice, nullptr, bias,
-                                                                 weights);
+  if (weights != nullptr)  // a wave chooses and weighs for a token, four tokens a workgroup; there is nothing to copy
+    moe_router_topk_kernel<float><<<(n_tokens + 3) / 4, 256, 4 * lds, stream>>>(logits, logits_stride, n_experts, top, nullptr, 0, 0, choice,
+                                                                                nullptr, bias, weights, n_tokens);
   else if (dtype == YK_F32)
     moe_router_topk_kernel<float><<<n_tokens, 256, lds, stream>>>(logits, logits_stride, n_experts, top, static_cast<const float*>(x), x_stride,
-                                                                  hidden, choice, static_cast<float*>(xs), bias, nullptr);
+                                                                  hidden, choice, static_cast<float*>(xs), bias, nullptr, n_tokens);
   else if (dtype == YK_BF16)
     moe_router_topk_kernel<bf16_t><<<n_tokens, 256, lds, stream>>>(logits, logits_stride, n_experts, top, static_cast<const bf16_t*>(x), x_stride,
-                                                                   hidden, choice, static_cast<bf16_t*>(xs), bias, nullptr);
+                                                                   hidden, choice, static_cast<bf16_t*>(xs), bias, nullptr, n_tokens);
   else
     return yk_fail("moe_router_topk: unsupported dtype");
   return yk_check_launch("moe_router_topk");

@@ -101,12 +101,43 @@ def mesolix_shape(width: int, vocab: int, heads: int, kv_heads: int, dim: int, k
     return {"architecture": "Mesolix", "vocab": vocab, "width": width, "max_positions": max_positions, "norm": {"eps": 1e-6}, "layers": layers}
 
 
+def bekedra_shape(width: int, vocab: int, heads: int, kv_heads: int, dim: int, experts: int, top: int, expert_ff: int,
+                  pattern=("attention_2", "attention", "attention", "attention_2"), loop=(1, 3, 2), original: int = 4096) -> dict:
+    """A Bekedra config.json of the given layer sizes: the mixers of ``pattern``, every layer with a mixture of experts,
+    the layers loop[0] .. loop[1] - 1 run loop[2] times in a row."""
+    first = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5, "q_temp": {"coef": 0.1, "every": 1024}}
+    second = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5, "softcap": 30.0,
+              "rot": {"base": 500000.0, "dims": dim // 2, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": original}}}
+    mlp = {"kind": "moe", "router": {"experts": experts, "top": top}, "expert": {"ff": expert_ff}}
+    layers = [{"type": kind, "mixer": dict(first if kind == "attention" else second), "mlp": dict(mlp)} for kind in pattern]
+    cfg = {"architecture": "Bekedra", "vocab": vocab, "width": width, "embedding": {"scale": float(width) ** 0.5}, "norm": {"eps": 1e-6},
+           "layers": layers}
+    if loop is not None:
+        cfg["loop"] = {"start": loop[0], "stop": loop[1], "times": loop[2]}
+    return cfg
+
+
+def layer_runs(design: dict) -> int:
+    """How many layers a token passes through (a looped stretch counts every pass)."""
+    loop = design.get("loop")
+    n = len(design["layers"])
+    return n if not loop else n + (loop["stop"] - loop["start"]) * (loop["times"] - 1)
+
+
 def llama_like(design: dict) -> dict:
     """The Llama configuration of equal size.  For Suranex: the same width, layer count, vocabulary
     and (first attention layer's) heads, a feed-forward as wide as what a token uses of the mixture
     (its top experts and the shared one).  For Nutavik: the same width, layer count, vocabulary and
     attention heads (keys as wide as its unrotated and rotated parts together, a quarter as many key
     heads), a gated feed-forward with as many weights as its dense one (two thirds as wide)."""
+    if design.get("architecture") == "Bekedra":
+        # the same width, vocabulary and heads, as many layers as a token passes through, a feed-forward with as many
+        # weights as what a token uses of the mixture (three matrices against an expert's two)
+        att = design["layers"][0]["mixer"]
+        f = next(layer["mlp"] for layer in design["layers"] if layer["mlp"] is not None)
+        inter = (2 * f["router"]["top"] * f["expert"]["ff"] // 3 + 255) // 256 * 256
+        return dict(LLAMA3_8B, hidden_size=design["width"], num_hidden_layers=layer_runs(design), num_attention_heads=att["heads"],
+                    num_key_value_heads=att["kv_heads"], head_dim=att["dim"], intermediate_size=inter, vocab_size=design["vocab"])
     if design.get("architecture") == "Mesolix":
         # the same width, layer count, vocabulary and (windowed attention's) heads; a feed-forward with as many
         # weights as the mean of what a token uses of the dense and the routed ones
@@ -147,6 +178,21 @@ def nutavik_like(design: dict) -> dict:
                          max(1, ssd["heads"] // 2), ssd["heads"], ssd["state"], ssd["vdim"], ff, repeats=max(1, len(design["layers"]) // 3))
 
 
+def mesolix_like(design: dict) -> dict:
+    """The Mesolix configuration of a Bekedra one's size: the same width, vocabulary, heads and experts (no shared
+    expert), as many layers as a token passes through (in threes), a window as long as the benchmark's prompts."""
+    att = design["layers"][0]["mixer"]
+    f = next(layer["mlp"] for layer in design["layers"] if layer["mlp"] is not None)
+    width = design["width"]
+    cfg = mesolix_shape(width, design["vocab"], att["heads"], att["kv_heads"], att["dim"], 512, 768 * width // 2048, 2048, 2 * att["heads"], 64, 128,
+                        max(1, att["heads"] // 8), 4 * width, f["router"]["experts"], f["router"]["top"], f["expert"]["ff"], f["expert"]["ff"],
+                        repeats=max(1, layer_runs(design) // 3))
+    for layer in cfg["layers"]:
+        if layer["mlp"] is not None and layer["mlp"]["kind"] == "moe":
+            layer["mlp"].pop("shared", None)
+    return cfg
+
+
 SURANEX_2K = suranex_shape(2048, 32768, 16, 4, 128, 1024, 2560, 10, 16, 2, 1024, 2048)
 SURANEX_4K = suranex_shape(4096, 65536, 32, 8, 128, 2048, 5120, 20, 32, 4, 1024, 4096, repeats=1)
 SURANEX_TINY = suranex_shape(64, 256, 4, 2, 16, 24, 96, 3, 4, 2, 32, 48, repeats=1)
@@ -156,6 +202,10 @@ NUTAVIK_TINY = nutavik_shape(64, 256, 4, 16, 8, 24, 32, 4, 2, 2, 16, 32, 96, rep
 MESOLIX_2K = mesolix_shape(2048, 32768, 16, 4, 128, 512, 768, 1024, 32, 64, 128, 2, 8192, 16, 2, 1024, 2048)
 MESOLIX_4K = mesolix_shape(4096, 65536, 32, 8, 128, 512, 1536, 2048, 64, 64, 128, 4, 16384, 32, 4, 1024, 4096, repeats=1)
 MESOLIX_TINY = mesolix_shape(64, 256, 4, 2, 16, 24, 32, 24, 4, 8, 16, 2, 96, 4, 2, 32, 48, bias_rows=8, max_positions=256, repeats=1, again=True)
+
+BEKEDRA_2K = bekedra_shape(2048, 32768, 16, 4, 128, 16, 2, 1024)
+BEKEDRA_4K = bekedra_shape(4096, 65536, 32, 8, 128, 32, 4, 1024, pattern=("attention_2", "attention"), loop=(1, 2, 2))
+BEKEDRA_TINY = bekedra_shape(64, 256, 4, 2, 16, 4, 2, 32, pattern=("attention_2", "attention", "attention_2"), loop=(0, 2, 2), original=32)
 
 # name -> (what to call it, config.json dictionary)
 SHAPES: Dict[str, Tuple[str, dict]] = {
@@ -174,6 +224,9 @@ SHAPES: Dict[str, Tuple[str, dict]] = {
     "mesolix-2k": ("Mesolix, width 2,048", MESOLIX_2K),
     "mesolix-4k": ("Mesolix, width 4,096", MESOLIX_4K),
     "mesolix-tiny": ("tiny Mesolix", MESOLIX_TINY),
+    "bekedra-2k": ("Bekedra, width 2,048", BEKEDRA_2K),
+    "bekedra-4k": ("Bekedra, width 4,096", BEKEDRA_4K),
+    "bekedra-tiny": ("tiny Bekedra", BEKEDRA_TINY),
 }
 
 

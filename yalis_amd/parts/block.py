@@ -69,15 +69,18 @@ class ParallelBlock(Block):
 
     def forward(self, residual, delta, ctx, site):
         h = self.norm.add_norm(residual, delta)
-        a = self.mixer.forward(h, ctx, site)
         if self.feed_forward is None:
-            return a
+            return self.mixer.forward(h, ctx, site)
+        # the feed-forward first: what it hands on is settled in tensors of its own before the mixer runs, and the
+        # mixer's output (possibly a product's unreduced slices in the library's workspace) is consumed right after
         f = self.feed_forward.forward(h, ctx)
         ops = self.mixer.rt.ops
         if not isinstance(f, ExpertRows):  # any other feed-forward: its output is one row a token
             f = ExpertRows(None, f.float().contiguous(), 1, 1.0)
-        if f.dense is not None:
-            a = ops.moe_combine(a, f.dense.float().contiguous(), 1, 1.0)
+        dense = None if f.dense is None else f.dense.float().contiguous()
+        a = self.mixer.forward(h, ctx, site)
+        if dense is not None:
+            a = ops.moe_combine(a, dense, 1, 1.0)
         return ops.moe_combine(a, f.rows, f.top, f.weight, row_weights=f.row_weights)
 
 
