@@ -68,8 +68,8 @@ CONFIGS = {
     # sizes of whole wavefronts (the matrix-core attention and grouped products in bfloat16); the loop begins with the
     # first layer and takes in all of them
     "wide": model(200, 128, 1e-6, 8.0, [
-        (sinked(4, 2, 64, 64, 0.125, softcap=20.0, rot=(32, 50000.0, 8.0, 1.0, 4.0, 64)), moe(8, 2, 64)),
-        (tempered(4, 2, 64, 0.125, 0.5, 64), moe(8, 2, 64)),
+        (sinked(4, 2, 64, 64, 0.125, softcap=25.0, rot=(32, 30000.0, 8.0, 1.0, 4.0, 64)), moe(8, 2, 64)),
+        (tempered(4, 2, 64, 0.125, 0.4, 48), moe(8, 2, 64)),
         (sinked(2, 1, 128, 128, 0.09, softcap=50.0, rot=(128, 10000.0)), moe(4, 2, 96)),
     ], loop=(0, 3, 2)),
 }
