@@ -588,7 +588,10 @@ def test_config_reader_and_spec():
         node[path[-1]] = value
         with pytest.raises(ConfigError, match=what):
             spec_from_config(bad)
-    for path in (("embedding",), ("layers", 0, "mixer", "scale"), ("norm", "eps")):
+    unscaled = copy.deepcopy(cfg)
+    del unscaled["embedding"]
+    assert spec_from_config(unscaled)[2].embedding.params["scale"] == 1.0
+    for path in (("embedding", "scale"), ("layers", 0, "mixer", "scale"), ("norm", "eps")):
         missing = copy.deepcopy(cfg)
         node = missing
         for key in path[:-1]:

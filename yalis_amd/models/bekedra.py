@@ -124,7 +124,8 @@ class BekedraConfig:
         r = KeyReader(raw)
         vocab, width = r.integer("vocab", minimum=1), r.integer("width", minimum=1)
         eps = KeyReader(r.mapping("norm"), where="config.json norm").number("eps", positive=True)
-        scale = KeyReader(r.mapping("embedding"), where="config.json embedding").number("scale", positive=True)
+        embedding = r.mapping("embedding", default=None)  # (left out: the rows as they are)
+        scale = 1.0 if embedding is None else KeyReader(embedding, where="config.json embedding").number("scale", positive=True)
         listed = r.raw_value("layers", None)
         if not isinstance(listed, list) or not listed:
             raise ConfigError("config.json: 'layers' must be a non-empty list")
