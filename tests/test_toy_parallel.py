@@ -25,7 +25,7 @@ BACKENDS = [
 ]
 
 
-class Toy3Config:
+class ToyParallelConfig:
     def __init__(self, raw):
         r = KeyReader(raw)
         r.taken.add("architectures")
@@ -40,7 +40,7 @@ class Toy3Config:
         return cls(raw)
 
 
-def build_toy3_spec(c: Toy3Config) -> ModelSpec:
+def build_toy_parallel_spec(c: ToyParallelConfig) -> ModelSpec:
     def rms(name):
         return PartSpec("rmsnorm", {"name": name, "size": c.hidden, "eps": c.eps, "unit_offset": False})
 
@@ -56,30 +56,30 @@ def build_toy3_spec(c: Toy3Config) -> ModelSpec:
         return PartSpec("dense_mlp", {"prefix": prefix, "hidden_size": c.hidden, "intermediate_size": c.inter, "activation": "relu2"})
 
     layers = (
-        LayerSpec.of("t3.0", "parallel", norm=rms("t3.0.n"), mixer=attn("t3.0.att"), feed_forward=dense("t3.0.ff")),
-        LayerSpec.of("t3.1", "prenorm", mixer_norm=layer_norm("t3.1.n1"), mixer=attn("t3.1.att"), feed_forward_norm=layer_norm("t3.1.n2"),
-                     feed_forward=dense("t3.1.ff")),
-        LayerSpec.of("t3.2", "parallel", norm=rms("t3.2.n"), mixer=attn("t3.2.att")),
+        LayerSpec.of("tp.0", "parallel", norm=rms("tp.0.n"), mixer=attn("tp.0.att"), feed_forward=dense("tp.0.ff")),
+        LayerSpec.of("tp.1", "prenorm", mixer_norm=layer_norm("tp.1.n1"), mixer=attn("tp.1.att"), feed_forward_norm=layer_norm("tp.1.n2"),
+                     feed_forward=dense("tp.1.ff")),
+        LayerSpec.of("tp.2", "parallel", norm=rms("tp.2.n"), mixer=attn("tp.2.att")),
     )
-    order = (RunEntry(0), RunEntry(1, added_row=("t3.rows", 1, 3)), RunEntry(2, added_row=("t3.rows", 2, 3)), RunEntry(0, added_row=("t3.rows", 0, 3)))
+    order = (RunEntry(0), RunEntry(1, added_row=("tp.rows", 1, 3)), RunEntry(2, added_row=("tp.rows", 2, 3)), RunEntry(0, added_row=("tp.rows", 0, 3)))
     return ModelSpec(
-        architecture="Toy3ForCausalLM", hidden_size=c.hidden, vocab_size=c.vocab, max_positions=256,
-        embedding=PartSpec("token_embedding", {"name": "t3.embed", "vocab_size": c.vocab, "hidden_size": c.hidden, "scale": 1.5}),
-        layers=layers, run_order=order, final_norm=rms("t3.final"),
-        head=PartSpec("lm_head", {"name": "t3.head", "tied_to": "t3.embed", "vocab_size": c.vocab, "hidden_size": c.hidden}),
+        architecture="ToyParallelForCausalLM", hidden_size=c.hidden, vocab_size=c.vocab, max_positions=256,
+        embedding=PartSpec("token_embedding", {"name": "tp.embed", "vocab_size": c.vocab, "hidden_size": c.hidden, "scale": 1.5}),
+        layers=layers, run_order=order, final_norm=rms("tp.final"),
+        head=PartSpec("lm_head", {"name": "tp.head", "tied_to": "tp.embed", "vocab_size": c.vocab, "hidden_size": c.hidden}),
     )
 
 
-register_architecture("Toy3ForCausalLM", Toy3Config, build_toy3_spec)
+register_architecture("ToyParallelForCausalLM", ToyParallelConfig, build_toy_parallel_spec)
 
-TOY3 = {"architectures": ["Toy3ForCausalLM"], "hidden_size": 72, "vocab_size": 97, "heads": 4, "kv_heads": 2, "head_dim": 16, "inner_size": 88,
+TOY_PARALLEL = {"architectures": ["ToyParallelForCausalLM"], "hidden_size": 72, "vocab_size": 97, "heads": 4, "kv_heads": 2, "head_dim": 16, "inner_size": 88,
         "eps": 1e-5, "theta": 10000.0}
 
 
-def toy3_plain(weights, tokens):
+def toy_parallel_plain(weights, tokens):
     """float64, whole sequence, dense masks."""
     W = {k: v.double() for k, v in weights.items()}
-    n, c = len(tokens), Toy3Config(TOY3)
+    n, c = len(tokens), ToyParallelConfig(TOY_PARALLEL)
     pos = torch.arange(n, dtype=torch.float64)
 
     def rms(x, name):
@@ -112,23 +112,23 @@ def toy3_plain(weights, tokens):
         a = torch.relu(h @ W[p + ".up_proj.weight"].T)
         return (a * a) @ W[p + ".down_proj.weight"].T
 
-    x = W["t3.embed"][torch.tensor(tokens)] * 1.5
-    h = rms(x, "t3.0.n")
-    x = x + attn(h, "t3.0.att") + dense(h, "t3.0.ff")
-    x = x + W["t3.rows"][1]
-    x = x + attn(layer_norm(x, "t3.1.n1"), "t3.1.att")
-    x = x + dense(layer_norm(x, "t3.1.n2"), "t3.1.ff")
-    x = x + W["t3.rows"][2]
-    x = x + attn(rms(x, "t3.2.n"), "t3.2.att")
-    x = x + W["t3.rows"][0]
-    h = rms(x, "t3.0.n")
-    x = x + attn(h, "t3.0.att") + dense(h, "t3.0.ff")
-    return rms(x, "t3.final") @ W["t3.embed"].T
+    x = W["tp.embed"][torch.tensor(tokens)] * 1.5
+    h = rms(x, "tp.0.n")
+    x = x + attn(h, "tp.0.att") + dense(h, "tp.0.ff")
+    x = x + W["tp.rows"][1]
+    x = x + attn(layer_norm(x, "tp.1.n1"), "tp.1.att")
+    x = x + dense(layer_norm(x, "tp.1.n2"), "tp.1.ff")
+    x = x + W["tp.rows"][2]
+    x = x + attn(rms(x, "tp.2.n"), "tp.2.att")
+    x = x + W["tp.rows"][0]
+    h = rms(x, "tp.0.n")
+    x = x + attn(h, "tp.0.att") + dense(h, "tp.0.ff")
+    return rms(x, "tp.final") @ W["tp.embed"].T
 
 
 def make_runner(device, dtype, num_pages):
     eng = EngineConfig(page_size=16, num_pages=num_pages, max_num_seqs=4, max_model_len=192, dtype=dtype, device=device)
-    model = build_model(TOY3, eng, ops=RefOps() if device == "cpu" else None)
+    model = build_model(TOY_PARALLEL, eng, ops=RefOps() if device == "cpu" else None)
     wd = torch.float32 if dtype == "float32" else torch.bfloat16
     weights = dict(random_tensors(model.tensor_specs(), 11, wd))
     model.load({k: v.to(device) for k, v in weights.items()})
@@ -139,12 +139,12 @@ def make_runner(device, dtype, num_pages):
 @pytest.mark.parametrize("mode", ["whole", "tail", "portions", "mixed"])
 def test_toy_model_replays(backend, mode):
     device, dtype = backend
-    reqs = C.make_requests({"vocab_size": TOY3["vocab_size"]}, [50, 21, 77, 9, 40], seed=6)
+    reqs = C.make_requests({"vocab_size": TOY_PARALLEL["vocab_size"]}, [50, 21, 77, 9, 40], seed=6)
     steps = {"whole": C.trace_whole, "tail": lambda r: C.trace_tail(r, tail=10), "portions": C.trace_portions, "mixed": C.trace_mixed}[mode](reqs)
     n_pages = C.pages_needed(steps, reqs, 16)
     runner, weights = make_runner(device, dtype, n_pages)
-    assert "t3.rows" in runner.model.tensor_specs() and len(runner.model.sites) == 4
-    want = {rid: toy3_plain(weights, toks).float() for rid, toks in reqs.items()}
+    assert "tp.rows" in runner.model.tensor_specs() and len(runner.model.sites) == 4
+    want = {rid: toy_parallel_plain(weights, toks).float() for rid, toks in reqs.items()}
     got, _ = C.run_trace(runner, steps)
     if dtype == "bfloat16":
         for rid, w in want.items():  # against the unrounded implementation: bfloat16's eight bits over four layer runs
